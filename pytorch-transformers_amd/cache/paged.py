@@ -24,7 +24,8 @@ wholly behind its window back to its pool as a sequence grows (their places in t
 layer that is zeroed when a slot is handed out.
 
 The K pool has the layout ``[layer, page, kv_head, page_size, head_dim]``, the V pool
-``[layer, page, kv_head, head_dim, page_size]``.
+``[layer, page, kv_head, head_dim, page_size]``.  A group with ``values=False`` has no V pool: its layers keep one
+row per token (a latent that keys and values are both made from) and read it as either.
 """
 from __future__ import annotations
 
@@ -66,8 +67,9 @@ class _Group:
             # (one page more than sequences can hold: the scratch page of padding rows)
             self.k = torch.zeros((spec.num_layers, num_pages + 1, spec.kv_heads, page_size, spec.head_dim),
                                  dtype=dtype, device=device)
-            self.v = torch.zeros((spec.num_layers, num_pages + 1, spec.kv_heads, spec.head_dim, page_size),
-                                 dtype=dtype, device=device)
+            if spec.values:
+                self.v = torch.zeros((spec.num_layers, num_pages + 1, spec.kv_heads, spec.head_dim, page_size),
+                                     dtype=dtype, device=device)
         elif spec.kind == CACHE_STATE:
             sd = spec.state_dtype or torch.float32
             # (one row more than there are slots: the scratch slot of padding rows)
@@ -188,7 +190,7 @@ class PagedCache:
     # storage -----------------------------------------------------------
     def kv_layer(self, group: str, layer: int):
         g = self.groups[group]
-        return g.k[layer], g.v[layer]
+        return g.k[layer], (None if g.v is None else g.v[layer])
 
     def state_layer(self, group: str, layer: int) -> torch.Tensor:
         return self.groups[group].state[layer]
@@ -220,7 +222,7 @@ class PagedCache:
         total = 0
         for g in self.groups.values():
             if g.k is not None:
-                total += 2 * g.spec.num_layers * g.spec.kv_heads * g.spec.head_dim * g.k.element_size()
+                total += (2 if g.v is not None else 1) * g.spec.num_layers * g.spec.kv_heads * g.spec.head_dim * g.k.element_size()
         return total
 
     def check_consistent(self) -> None:

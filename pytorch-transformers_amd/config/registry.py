@@ -76,7 +76,13 @@ class AutoConfig:
     def from_dict(d: dict, **overrides) -> ModelConfig:
         d = dict(d)
         if "model_type" not in d:
-            raise ConfigError("config.json has no 'model_type' key; cannot choose an architecture")
+            # a file that names its design under "architecture" (or the first of "architectures") instead
+            named = d.get("architecture") or (d.get("architectures") or [None])[0]
+            if isinstance(named, str) and (resolve_alias(named) in _REGISTRY or named.lower() in _REGISTRY):
+                d["model_type"] = resolve_alias(named) if resolve_alias(named) in _REGISTRY else named.lower()
+        if "model_type" not in d:
+            raise ConfigError("config.json has no 'model_type' key (and names no known 'architecture'); cannot "
+                              "choose an architecture")
         d["model_type"] = resolve_alias(d["model_type"])
         cls, _ = lookup(d["model_type"])
         return cls.from_dict(d, **overrides)

@@ -14,7 +14,7 @@
 
 #include <stdint.h>
 
-#define PTA_ABI_VERSION 9
+#define PTA_ABI_VERSION 10
 
 #ifdef __cplusplus
 extern "C" {
@@ -236,6 +236,42 @@ int pta_argmax(int* out_tok, const float* logits, int R, int V, void* stream);
 
 // host function: the uniform number in [0, 1) that pta_sample draws for (seed, sequence, step)
 float pta_philox_uniform(uint64_t seed, uint32_t seq, uint32_t step);
+
+// ---- a residual stream held in 32-bit (rms_stream.hip) ------------------------------------------------------
+// v = x (* silu(gate)); n = v / sqrt(mean(v^2) + eps) * (offset + w), each of `groups` equal parts of a row by its
+// own mean; out = residual + mult * n where residual is given, else n; written as 32-bit (out_wide) and / or in the
+// compute type (out_narrow).  x is 32-bit if x_wide, else of the compute type; gate is of the compute type;
+// x_ld / gate_ld: distance of their rows; rows (may be null) picks the source rows.
+int pta_rmsnorm(void* out_narrow, float* out_wide, const void* x, int x_wide, long x_ld, const void* gate, long gate_ld,
+                const int* rows, const float* w, float offset, int groups, float eps, const float* residual, float mult,
+                int M, int H, int dtype, void* stream);
+// out[i] = sum_j coef[j] * planes[j * plane + i], j in order; 32-bit and / or compute type
+int pta_depth_mix(float* out_wide, void* out_narrow, const float* planes, long plane, const float* coef, int count,
+                  long n, int dtype, void* stream);
+int pta_widen(float* out, const void* in, long n, int dtype, void* stream);
+int pta_scale_f32(float* x, float f, long n, void* stream);
+
+// ---- layers with a state of fixed size per sequence (recurrent.hip) ----------------------------------------------
+int pta_gated_scan(void* y, const void* zxg, long ld, const float* bz, const float* bx, float* state, long state_ld,
+                   const int* cu_tokens, const int* seq_slot, int n_seqs, int W, int dtype, void* stream);
+int pta_conv_silu(float* out, const void* in, long ld, const float* w, const float* b, float* tail, long tail_ld,
+                  const int* cu_tokens, const int* token_seq, const int* seq_slot, int n_seqs, int M, int C, int K,
+                  int dtype, void* stream);
+int pta_ssm_scan(float* y, const float* xbc, const void* dt_in, long dt_ld, const float* dt_bias, const float* A_log,
+                 const float* Dp, float* state, long state_ld, const int* cu_tokens, const int* seq_slot, int n_seqs,
+                 int heads, int P, int N, int G, int dtype, void* stream);
+
+// ---- attention over a cache of latents (attn_latent.hip) ----------------------------------------------------------
+int pta_attn_latent_sizes_ok(int H, int dn, int dr, int R);
+int pta_latent_prep(float* q_full, void* k_pool, const void* proj, long ld, const float* w_norm, float eps,
+                    const PtaRotation* rot, const int* token_pos, const int* token_seq, const int* block_table,
+                    int bt_stride, int M, int H, int dn, int dr, int R, int write_cache, int dtype, void* stream);
+int pta_head_project(void* out, int out_wide, long out_ld, long out_head, const void* in, int in_wide, long in_ld,
+                     long in_head, const void* w, long w_head, long w_o, long w_k, int M, int H, int K, int O,
+                     int dtype, void* stream);
+int pta_attn_latent(float* out, const float* q, const void* k_pool, const int* block_table, int bt_stride,
+                    const int* token_seq, const int* token_pos, int M, int H, int R, int dr, float scale, int dtype,
+                    void* stream);
 
 #ifdef __cplusplus
 }

@@ -23,7 +23,7 @@ import torch
 from .. import host, tuning
 from ..cache.paged import PagedCache
 from ..config.registry import AutoConfig, lookup
-from ..parts.base import ResidualSum, StepContext, as_tensor
+from ..parts.base import ResidualSum, StepContext, WideResidual, as_tensor
 from ..weights.loader import load_weights
 from ..weights.random_init import random_tensors
 from .spec import ModelSpec
@@ -449,6 +449,8 @@ class CausalLM:
             block = blocks[call.block]
             if isinstance(x, ResidualSum) and not getattr(block, "accepts_sum", False):
                 x = x.tensor()
+            elif isinstance(x, WideResidual) and not getattr(block, "accepts_wide", False):
+                x = x.narrow
             x = block.forward(x, ctx, call)
             if self.layer_hook is not None:
                 self.layer_hook(i, as_tensor(x))  # a sum that is not formed yet is formed for the hook alone
@@ -457,6 +459,9 @@ class CausalLM:
         norm = self.spec.final_norm
         if isinstance(x, ResidualSum) and norm is not None and hasattr(norm, "forward_sum"):
             h = norm.forward_sum(x, rows=logit_rows, want_x=False)[1]
+        elif isinstance(x, WideResidual):  # a stream kept in 32-bit: the norm reads that side
+            h = norm.forward_wide(x, rows=logit_rows) if norm is not None and hasattr(norm, "forward_wide") else (
+                norm.forward(x.narrow, rows=logit_rows) if norm is not None else x.narrow.index_select(0, logit_rows.long()))
         else:
             x = as_tensor(x)
             h = norm.forward(x, rows=logit_rows) if norm is not None else x.index_select(0, logit_rows.long())

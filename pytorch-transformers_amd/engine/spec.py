@@ -52,6 +52,8 @@ class CacheGroupSpec:
     kv_heads: int = 0
     head_dim: int = 0
     window: Optional[int] = None
+    #: False: the group keeps no value pool (its layers read their values out of the key rows)
+    values: bool = True
     state_shape: Tuple[int, ...] = ()
     state_dtype: Any = None  # None: 32-bit float
 

@@ -24,7 +24,7 @@ QKV_LAYOUT_CODES = {"grouped": 0, "tail": 1, "interleaved": 2}
 ACT_CODES = {None: 0, "none": 0, "linear": 0, "gelu": 1, "gelu_python": 1, "gelu_new": 2, "gelu_pytorch_tanh": 2,
              "gelu_fast": 2, "gelu_accurate": 2, "quick_gelu": 3, "relu": 4, "relu2": 5, "relu6": 6, "silu": 7, "swish": 7,
              "sigmoid": 8, "tanh": 9, "leaky_relu": 10, "mish": 11, "gelu_10": 12, "laplace": 13}
-ABI_VERSION = 9
+ABI_VERSION = 10
 PAIRING_CODES = {"half": 0, "interleaved": 1}  # PtaPairing: elements (i, i + rotary_dim / 2) or (2i, 2i + 1)
 BIAS_OF_CODES = {"key": 0, "distance": 1}  # PtaBiasOf: the slope times the key's position, or times key - query position
 
@@ -1006,4 +1006,262 @@ def gemm_skinny_bf16(x: torch.Tensor, w: torch.Tensor, bias=None, act=None, add1
     out = torch.empty((M, N), dtype=torch.float32 if out_f32 else torch.bfloat16, device=x.device)
     _call("pta_gemm_skinny_bf16", _ptr(out), _ptr(x), _ptr(w), _ptr(bias), _ptr(add1), _ptr(add2), M, N, K,
           ACT_CODES[act], int(out_f32), int(variant), int(waves), _stream())
+    return out
+
+
+# ---- a residual stream held in 32-bit ---------------------------------------------------------------------------
+def _rows_of(t: torch.Tensor, name: str, cols: int, dtype=None):
+    """Check a matrix whose rows may lie apart (a block of columns of a wider one) and return its row distance."""
+    if not isinstance(t, torch.Tensor) or not t.is_cuda or t.dim() != 2 or t.shape[1] != cols or t.stride(1) != 1:
+        raise KernelError(f"{name} must be a GPU matrix [rows, {cols}] with adjacent columns, got "
+                          f"{tuple(getattr(t, 'shape', ()))} strides {getattr(t, 'stride', lambda: None)()}")
+    if dtype is not None and t.dtype != dtype:
+        raise KernelError(f"{name} must be {dtype}, got {t.dtype}")
+    return int(t.stride(0)) if t.shape[0] > 1 else max(int(t.stride(0)), cols)
+
+
+def rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float, dtype: torch.dtype, *, offset: float = 0.0, groups: int = 1,
+            gate: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None,
+            residual: Optional[torch.Tensor] = None, mult: float = 1.0, want_wide: bool = False, want_narrow: bool = True,
+            out_wide: Optional[torch.Tensor] = None):
+    """RMS norm in 32-bit: ``n = v / sqrt(mean(v^2) + eps) * (offset + w)`` with ``v = x`` or ``x * silu(gate)``,
+    each of ``groups`` equal parts of a row by its own mean square; with ``residual`` (32-bit) the result is
+    ``residual + mult * n``.  ``x`` is 32-bit or of the compute type ``dtype`` and its rows may lie apart, as may
+    the gate's.  Returns ``(narrow, wide)``: the result in ``dtype`` and in 32-bit (each None unless wanted;
+    ``out_wide``: where to write the 32-bit result).  In a 32-bit model the two are one tensor."""
+    H = w.numel()
+    _need(w, "weight", torch.float32, (H,))
+    x_wide = x.dtype == torch.float32
+    if not x_wide and x.dtype != dtype:
+        raise KernelError(f"x must be 32-bit or {dtype}, got {x.dtype}")
+    x_ld = _rows_of(x, "x", H)
+    gate_ld = 0 if gate is None else _rows_of(gate, "gate", H, dtype)
+    if rows is not None:
+        _need(rows, "rows", torch.int32)
+        M = rows.numel()
+    else:
+        M = x.shape[0]
+    if gate is not None and gate.shape[0] != x.shape[0]:
+        raise KernelError("gate and x differ in their number of rows")
+    if residual is not None:
+        _need(residual, "residual", torch.float32, (x.shape[0], H))
+    if H % groups:
+        raise KernelError(f"{H} features do not split into {groups} equal groups")
+    f32 = dtype == torch.float32
+    if out_wide is not None:
+        _need(out_wide, "out_wide", torch.float32, (M, H))
+        want_wide = True
+    elif want_wide or (f32 and want_narrow):
+        out_wide = torch.empty((M, H), dtype=torch.float32, device=x.device)
+    narrow = None
+    if want_narrow and not f32:
+        narrow = torch.empty((M, H), dtype=dtype, device=x.device)
+    if M:
+        _call("pta_rmsnorm", _ptr(narrow), _ptr(out_wide), _ptr(x), int(x_wide), ctypes.c_long(x_ld), _ptr(gate),
+              ctypes.c_long(gate_ld), _ptr(rows), _ptr(w), ctypes.c_float(offset), int(groups), ctypes.c_float(eps),
+              _ptr(residual), ctypes.c_float(mult), M, H, dtype_code(dtype), _stream())
+    if f32:
+        return (out_wide if want_narrow else None), (out_wide if want_wide else None)
+    return narrow, (out_wide if want_wide else None)
+
+
+def depth_mix(planes: torch.Tensor, coef: torch.Tensor, count: int, dtype: torch.dtype):
+    """``sum_j coef[j] * planes[j]`` over the first ``count`` planes of ``[planes, rows, features]`` (32-bit), added
+    in that order; returns ``(narrow, wide)``: the sum in ``dtype`` and in 32-bit (one tensor in a 32-bit model)."""
+    _need(planes, "planes", torch.float32)
+    if planes.dim() != 3 or not (0 < count <= planes.shape[0]):
+        raise KernelError(f"planes must be [at least {count}, rows, features], got {tuple(planes.shape)}")
+    _need(coef, "coef", torch.float32, (count,))
+    _, M, H = planes.shape
+    wide = torch.empty((M, H), dtype=torch.float32, device=planes.device)
+    narrow = None if dtype == torch.float32 else torch.empty((M, H), dtype=dtype, device=planes.device)
+    if M:
+        _call("pta_depth_mix", _ptr(wide), _ptr(narrow), _ptr(planes), ctypes.c_long(M * H), _ptr(coef), int(count),
+              ctypes.c_long(M * H), dtype_code(dtype), _stream())
+    return (wide if narrow is None else narrow), wide
+
+
+def widen(x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``x`` (compute type) as 32-bit, into ``out`` if given."""
+    _need(x, "x")
+    if out is None:
+        out = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+    _need(out, "out", torch.float32, tuple(x.shape))
+    if x.numel():
+        _call("pta_widen", _ptr(out), _ptr(x), ctypes.c_long(x.numel()), dtype_code(x.dtype), _stream())
+    return out
+
+
+def scale_(x: torch.Tensor, factor: float) -> torch.Tensor:
+    """In place: ``x *= factor`` (32-bit)."""
+    _need(x, "x", torch.float32)
+    if x.numel() and factor != 1.0:
+        _call("pta_scale_f32", _ptr(x), ctypes.c_float(factor), ctypes.c_long(x.numel()), _stream())
+    return x
+
+
+# ---- layers with a state of fixed size per sequence -------------------------------------------------------------
+def _need_state(state: torch.Tensor, row: int, name: str = "state") -> int:
+    """A state table ``[slots, >= row]`` in 32-bit whose rows may lie apart; returns the row distance."""
+    if not (isinstance(state, torch.Tensor) and state.is_cuda and state.dtype == torch.float32 and state.dim() == 2
+            and state.stride(1) == 1 and state.shape[1] >= row):
+        raise KernelError(f"{name} must be a 32-bit GPU table [slots, at least {row}] with adjacent columns")
+    return int(state.stride(0))
+
+
+def gated_scan(zxg: torch.Tensor, bz, bx, state: torch.Tensor, cu_tokens: torch.Tensor, seq_slot: torch.Tensor) -> torch.Tensor:
+    """The gated recurrence ``S = (1 - z) S + z c`` over every sequence's tokens of the step, from and into its row
+    of ``state`` ``[slots, W]``: ``zxg`` ``[tokens, 3 W]`` holds the gate's and the candidate's pre-activations
+    (biases ``bz``, ``bx`` still to add) and the output gate; returns ``S * silu(g)`` ``[tokens, W]``."""
+    if zxg.dim() != 2 or zxg.shape[1] % 3:
+        raise KernelError(f"zxg must be [tokens, 3 * width], got {tuple(zxg.shape)}")
+    M, W = zxg.shape[0], zxg.shape[1] // 3
+    ld = _rows_of(zxg, "zxg", 3 * W)
+    for name, b in (("bz", bz), ("bx", bx)):
+        if b is not None:
+            _need(b, name, torch.float32, (W,))
+    n = seq_slot.numel()
+    _need(seq_slot, "seq_slot", torch.int32, (n,))
+    _need(cu_tokens, "cu_tokens", torch.int32, (n + 1,))
+    state_ld = _need_state(state, W)
+    y = torch.empty((M, W), dtype=zxg.dtype, device=zxg.device)
+    if M:
+        _call("pta_gated_scan", _ptr(y), _ptr(zxg), ctypes.c_long(ld), _ptr(bz), _ptr(bx), _ptr(state),
+              ctypes.c_long(state_ld), _ptr(cu_tokens), _ptr(seq_slot), n, W, dtype_code(zxg.dtype), _stream())
+    return y
+
+
+def conv_silu(x: torch.Tensor, w: torch.Tensor, b, tail: torch.Tensor, cu_tokens, token_seq, seq_slot) -> torch.Tensor:
+    """``silu`` of a causal convolution per channel over each sequence's tokens: ``w`` ``[channels, taps]`` (the last
+    tap is the token's own), ``b`` ``[channels]`` or None; ``tail`` ``[slots, (taps - 1) * channels]`` holds every
+    sequence's last inputs from before the step and is moved on.  ``x`` ``[tokens, channels]`` may be a block of
+    columns; the result is 32-bit."""
+    C, K = w.shape
+    _need(w, "w", torch.float32)
+    if b is not None:
+        _need(b, "b", torch.float32, (C,))
+    M = x.shape[0]
+    ld = _rows_of(x, "x", C)
+    n = seq_slot.numel()
+    _need(seq_slot, "seq_slot", torch.int32, (n,))
+    _need(cu_tokens, "cu_tokens", torch.int32, (n + 1,))
+    _need(token_seq, "token_seq", torch.int32, (M,))
+    tail_ld = _need_state(tail, (K - 1) * C, "tail")
+    out = torch.empty((M, C), dtype=torch.float32, device=x.device)
+    if M:
+        _call("pta_conv_silu", _ptr(out), _ptr(x), ctypes.c_long(ld), _ptr(w), _ptr(b), _ptr(tail), ctypes.c_long(tail_ld),
+              _ptr(cu_tokens), _ptr(token_seq), _ptr(seq_slot), n, M, C, K, dtype_code(x.dtype), _stream())
+    return out
+
+
+def ssm_scan(xbc: torch.Tensor, dt: torch.Tensor, dt_bias, a_log, d_skip, state: torch.Tensor, cu_tokens, seq_slot,
+             heads: int, head_dim: int, state_rows: int, groups: int) -> torch.Tensor:
+    """The state-space recurrence per head over every sequence's tokens, from and into its row of ``state``
+    ``[slots, heads * state_rows * head_dim]``: ``xbc`` ``[tokens, heads * head_dim + 2 * groups * state_rows]``
+    (32-bit: inputs, then B, then C per group), ``dt`` ``[tokens, heads]`` (compute type, may be a block of
+    columns; softplus and ``dt_bias`` are applied here).  Returns y ``[tokens, heads * head_dim]`` in 32-bit."""
+    inner = heads * head_dim
+    C = inner + 2 * groups * state_rows
+    M = xbc.shape[0]
+    _need(xbc, "xbc", torch.float32, (M, C))
+    dt_ld = _rows_of(dt, "dt", heads)
+    for name, t in (("dt_bias", dt_bias), ("A_log", a_log), ("D", d_skip)):
+        _need(t, name, torch.float32, (heads,))
+    n = seq_slot.numel()
+    _need(seq_slot, "seq_slot", torch.int32, (n,))
+    _need(cu_tokens, "cu_tokens", torch.int32, (n + 1,))
+    state_ld = _need_state(state, heads * state_rows * head_dim)
+    y = torch.empty((M, inner), dtype=torch.float32, device=xbc.device)
+    if M:
+        _call("pta_ssm_scan", _ptr(y), _ptr(xbc), _ptr(dt), ctypes.c_long(dt_ld), _ptr(dt_bias), _ptr(a_log), _ptr(d_skip),
+              _ptr(state), ctypes.c_long(state_ld), _ptr(cu_tokens), _ptr(seq_slot), n, heads, head_dim, state_rows,
+              groups, dtype_code(dt.dtype), _stream())
+    return y
+
+
+# ---- attention over a cache of latents ---------------------------------------------------------------------------
+def latent_sizes_problem(heads: int, dim: int, rot_dim: int, rank: int) -> Optional[str]:
+    """None if the latent attention launches take these sizes, else why not."""
+    lib = load_library()
+    if lib.pta_attn_latent_sizes_ok(int(heads), int(dim), int(rot_dim), int(rank)) == 0:
+        return None
+    return lib.pta_last_error().decode("utf-8", "replace")
+
+
+def latent_prep(proj: torch.Tensor, w_norm: torch.Tensor, eps: float, inv_freq, cs_scale: float, rotary_dim, pairing: str,
+                token_pos, token_seq, block_table, k_pool, heads: int, dim: int, rot_dim: int, rank: int,
+                write_cache: bool = True) -> torch.Tensor:
+    """From ``proj`` ``[tokens, heads * (dim + rot_dim) + rank + rot_dim]`` (the queries, then the down-projection):
+    the normed latent and the rotated shared key part go into the token's cache row ``[rank + rot_dim]``; returns
+    the queries' frame ``[tokens, heads, rank + rot_dim]`` in 32-bit with the rotated parts filled in (the first
+    ``rank`` of each head are for ``head_project``)."""
+    M = proj.shape[0]
+    cols = heads * (dim + rot_dim) + rank + rot_dim
+    ld = _rows_of(proj, "proj", cols)
+    _need(w_norm, "w_norm", torch.float32, (rank,))
+    _need(token_pos, "token_pos", torch.int32, (M,))
+    _need(token_seq, "token_seq", torch.int32, (M,))
+    _need(block_table, "block_table", torch.int32)
+    D = rank + rot_dim
+    _need(k_pool, "k_pool", proj.dtype)
+    if k_pool.dim() != 4 or tuple(k_pool.shape[1:]) != (1, 64, D):
+        raise KernelError(f"k_pool must be [pages, 1, 64, {D}], got {tuple(k_pool.shape)}")
+    rot = _rotation_arg(inv_freq, cs_scale, rot_dim, block_table.shape[0], rotary_dim, pairing) if rot_dim else None
+    q_full = torch.empty((M, heads, D), dtype=torch.float32, device=proj.device)
+    if M:
+        _call("pta_latent_prep", _ptr(q_full), _ptr(k_pool), _ptr(proj), ctypes.c_long(ld), _ptr(w_norm),
+              ctypes.c_float(eps), rot, _ptr(token_pos), _ptr(token_seq), _ptr(block_table), block_table.shape[1], M,
+              heads, dim, rot_dim, rank, int(write_cache), dtype_code(proj.dtype), _stream())
+    return q_full
+
+
+def head_project(x: torch.Tensor, x_head: int, w: torch.Tensor, heads: int, K: int, O: int, transposed: bool,
+                 out: Optional[torch.Tensor] = None, out_head: Optional[int] = None, out_dtype=None) -> torch.Tensor:
+    """A product per head: ``out[t, h, :O] = W_h x[t, h, :K]``.  ``x`` is ``[tokens, >= heads * x_head]`` (rows may
+    lie apart; head h starts at column ``h * x_head``), 32-bit or of w's type.  ``w`` is ``[heads * O, K]``
+    (``transposed=False``: head h's rows are its outputs) or ``[heads * K, O]`` (``transposed=True``: head h's rows
+    are its inputs, the product is with the transpose).  The result goes to ``out`` ``[tokens, >= heads * out_head]``
+    if given (32-bit or w's type), else to a new ``[tokens, heads * O]`` of ``out_dtype`` (default w's type)."""
+    _need(w, "w")
+    if tuple(w.shape) != ((heads * K, O) if transposed else (heads * O, K)):
+        raise KernelError(f"w {tuple(w.shape)} does not hold {heads} heads of {O} x {K}"
+                          + (" (transposed)" if transposed else ""))
+    M = x.shape[0]
+    if x.dim() != 2 or x.stride(1) != 1 or not x.is_cuda or x.shape[1] < (heads - 1) * x_head + K:
+        raise KernelError(f"x {tuple(x.shape)} does not hold {heads} heads of {K} elements {x_head} apart")
+    if x.dtype not in (torch.float32, w.dtype):
+        raise KernelError(f"x must be 32-bit or {w.dtype}, got {x.dtype}")
+    if out is None:
+        out_head = O
+        out = torch.empty((M, heads * O), dtype=out_dtype or w.dtype, device=x.device)
+    if out.dim() != 2 or out.stride(1) != 1 or out.shape[0] != M or out.shape[1] < (heads - 1) * out_head + O:
+        raise KernelError(f"out {tuple(out.shape)} does not hold {heads} heads of {O} elements {out_head} apart")
+    if out.dtype not in (torch.float32, w.dtype):
+        raise KernelError(f"out must be 32-bit or {w.dtype}, got {out.dtype}")
+    w_head, w_o, w_k = (K * O, 1, O) if transposed else (O * K, K, 1)
+    if M:
+        _call("pta_head_project", _ptr(out), int(out.dtype == torch.float32), ctypes.c_long(out.stride(0)),
+              ctypes.c_long(out_head), _ptr(x), int(x.dtype == torch.float32), ctypes.c_long(x.stride(0)),
+              ctypes.c_long(x_head), _ptr(w), ctypes.c_long(w_head), ctypes.c_long(w_o), ctypes.c_long(w_k), M, heads, K,
+              O, dtype_code(w.dtype), _stream())
+    return out
+
+
+def attn_latent(q_full: torch.Tensor, k_pool: torch.Tensor, block_table, token_seq, token_pos, rank: int,
+                scale: float) -> torch.Tensor:
+    """Causal attention of every token over its sequence's cache rows ``[rank + rot_dim]``, whose first ``rank``
+    elements are also the values: ``q_full`` ``[tokens, heads, rank + rot_dim]`` (32-bit) -> ``[tokens, heads,
+    rank]`` (32-bit)."""
+    _need(q_full, "q_full", torch.float32)
+    M, H, D = q_full.shape
+    if k_pool.dim() != 4 or tuple(k_pool.shape[1:]) != (1, 64, D) or not k_pool.is_cuda or not k_pool.is_contiguous():
+        raise KernelError(f"k_pool must be [pages, 1, 64, {D}], got {tuple(k_pool.shape)}")
+    _need(block_table, "block_table", torch.int32)
+    _need(token_seq, "token_seq", torch.int32, (M,))
+    _need(token_pos, "token_pos", torch.int32, (M,))
+    out = torch.empty((M, H, rank), dtype=torch.float32, device=q_full.device)
+    if M:
+        _call("pta_attn_latent", _ptr(out), _ptr(q_full), _ptr(k_pool), _ptr(block_table), block_table.shape[1],
+              _ptr(token_seq), _ptr(token_pos), M, H, int(rank), D - int(rank), ctypes.c_float(scale),
+              dtype_code(k_pool.dtype), _stream())
     return out

@@ -24,6 +24,8 @@ positions      ``rotation() -> (inv_freq or None, scale)`` for queries and keys,
                optionally ``rotation_for(ctx) -> (table, scale)`` where the table may
                have a row per sequence of the step (frequencies that follow a length)
 block          ``forward(x, ctx, call) -> x``: the arrangement of the above
+stream         what a block does to the residual stream between layers (a weighted
+               sum of the streams that earlier layers left: ``parts.depth``)
 =============  ==================================================================
 
 Optional: a mixer or feed-forward that sets ``can_defer = True`` and is called with
@@ -46,7 +48,7 @@ import torch
 
 from ..engine.spec import TensorSpec
 
-_KINDS = ("mixer", "feed_forward", "norm", "positions", "block")
+_KINDS = ("mixer", "feed_forward", "norm", "positions", "block", "stream")
 _TABLE: Dict[str, Dict[str, type]] = {k: {} for k in _KINDS}
 
 
@@ -137,8 +139,21 @@ class ResidualSum:
         return ops.layernorm_sum(self.kernel_terms(), self.features)[0]
 
 
+class WideResidual:
+    """The residual stream held in 32-bit (``wide``) beside the same values in the model's compute type
+    (``narrow``), which is what the next matrix product reads; in a 32-bit model the two are one tensor.
+    ``history``: what a block that mixes the streams of earlier layers keeps for the step (see
+    ``parts.depth.DepthMix``), handed on from block to block."""
+
+    def __init__(self, wide: torch.Tensor, narrow: torch.Tensor, history=None):
+        self.wide, self.narrow, self.history = wide, narrow, history
+
+
 def as_tensor(x):
-    """A tensor from what a part may hand on: a tensor, a ``PartialProduct`` or a ``ResidualSum``."""
+    """A tensor from what a part may hand on: a tensor, a ``PartialProduct``, a ``ResidualSum`` or a
+    ``WideResidual`` (its 32-bit side)."""
+    if isinstance(x, WideResidual):
+        return x.wide
     if isinstance(x, PartialProduct):
         return ResidualSum([x]).tensor()
     if isinstance(x, ResidualSum):

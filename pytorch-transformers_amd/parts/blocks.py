@@ -17,7 +17,7 @@ from typing import Optional, Sequence
 
 import torch
 
-from .base import Part, ResidualSum, StepContext, register_part
+from .base import Part, ResidualSum, StepContext, WideResidual, as_tensor, register_part
 from .linear import Linear, PendingProjection
 
 
@@ -126,5 +126,67 @@ class SequentialBlock(Part):
         return self.feed_forward.forward(m, ctx, add1=r)
 
 
+class PostNormBlock(Part):
+    """``x <- x + m * norm_mixer(mixer(x))``, then ``x <- x + m * norm_ffn(ffn(x))``: the sublayers read the stream
+    itself and the norm stands on each sublayer's output; ``m`` is a constant.  The stream is kept in 32-bit
+    whatever the compute type (``WideResidual``): a sublayer reads its copy in the compute type, the norm, the
+    scaling and the addition are one 32-bit launch that also writes that copy for the next sublayer.
+    ``feed_forward`` may be None (a layer of the mixer alone).  With ``depth_mix`` (``parts.depth.DepthMix``) the
+    block's result is kept as the next of the step's streams and what goes on is their weighted sum."""
+
+    accepts_sum = False
+    accepts_wide = True
+
+    def __init__(self, mixer: Part, feed_forward: Optional[Part], norm_mixer: Part, norm_ffn: Optional[Part],
+                 residual_mult: float = 1.0, depth_mix: Optional[Part] = None):
+        if (feed_forward is None) != (norm_ffn is None):
+            raise ValueError("a feed-forward and its norm come together or not at all")
+        self.mixer, self.feed_forward, self.norm_mixer, self.norm_ffn = mixer, feed_forward, norm_mixer, norm_ffn
+        self.residual_mult = float(residual_mult)
+        self.depth_mix = depth_mix
+
+    def children(self) -> Sequence[Part]:
+        return tuple(p for p in (self.norm_mixer, self.norm_ffn, self.mixer, self.feed_forward, self.depth_mix)
+                     if p is not None)
+
+    def after_load(self) -> None:
+        for part in (self.mixer, self.feed_forward):
+            if part is not None and hasattr(part, "after_load"):
+                part.after_load()
+
+    def _enter(self, x, ctx: StepContext) -> WideResidual:
+        """The stream as this block wants it; the first block of a model is given the embedding's plain tensor."""
+        from .. import ops
+
+        if isinstance(x, WideResidual):
+            return x
+        x = as_tensor(x)
+        history = None
+        if self.depth_mix is not None:
+            history = self.depth_mix.new_history(x.shape[0], x.shape[1], x.device)
+            wide = ops.widen(x, history.next_plane())
+        else:
+            wide = x if x.dtype == torch.float32 else ops.widen(x)
+        return WideResidual(wide, x if x.dtype == ctx.dtype else wide, history)
+
+    def forward(self, x, ctx: StepContext, call):
+        x = self._enter(x, ctx)
+        last = self.feed_forward is None
+        history = x.history
+        keep = history.next_plane() if (history is not None and self.depth_mix is not None) else None
+        mixed = self.mixer.forward(x.narrow, ctx, call)
+        narrow, wide = self.norm_mixer.apply(mixed, ctx.dtype, residual=x.wide, mult=self.residual_mult,
+                                             want_wide=True, want_narrow=not last or keep is None,
+                                             out_wide=keep if last else None)
+        if not last:
+            out = self.feed_forward.forward(narrow, ctx)
+            narrow, wide = self.norm_ffn.apply(out, ctx.dtype, residual=wide, mult=self.residual_mult, want_wide=True,
+                                               want_narrow=keep is None, out_wide=keep)
+        if keep is not None:
+            narrow, wide = self.depth_mix.forward(history, ctx.dtype)
+        return WideResidual(wide, narrow, history)
+
+
+register_part("block", "post_norm", PostNormBlock)
 register_part("block", "parallel", ParallelBlock)
 register_part("block", "sequential", SequentialBlock)

@@ -15,13 +15,16 @@ from .linear import Linear, PendingProjection
 
 class DenseFeedForward(Part):
     def __init__(self, name: str, hidden_size: int, ffn_size: int, bias: bool, activation: str = "gelu",
-                 up_name: str = "dense_h_to_4h", down_name: str = "dense_4h_to_h"):
+                 up_name: str = "dense_h_to_4h", down_name: str = "dense_4h_to_h", bare_names: bool = False):
+        """``bare_names``: the weight file holds the matrices as ``name.up_name`` and ``name.down_name`` themselves,
+        with no ``.weight`` behind them."""
         if activation not in ops.ACT_CODES:
             raise ValueError(f"activation {activation!r} is not built; built: {sorted(k for k in ops.ACT_CODES if k)}")
         self.name = name
         self.activation = activation
-        self.up = Linear(f"{name}.{up_name}", hidden_size, ffn_size, bias)
-        self.down = Linear(f"{name}.{down_name}", ffn_size, hidden_size, bias)
+        bare = (lambda n: n) if bare_names else (lambda n: None)
+        self.up = Linear(f"{name}.{up_name}", hidden_size, ffn_size, bias, weight_name=bare(f"{name}.{up_name}"))
+        self.down = Linear(f"{name}.{down_name}", ffn_size, hidden_size, bias, weight_name=bare(f"{name}.{down_name}"))
 
     def children(self) -> Sequence[Part]:
         return (self.up, self.down)

@@ -1,0 +1,91 @@
+"""Attention over a cache of latents: per token the cache holds one small vector c (``rank`` elements, the
+RMS-normed first rows of a down-projection) and one rotated key part (``rot_dim`` elements, the rest of it) that
+all heads share.  Per head the plain key is ``U_k c`` and the value ``U_v c``; the score of a query and a key is
+``(q_plain . k_plain + q_rot . k_rot) * scale``, softmax over the causal keys, output projection on the heads' values.
+
+The two expansions are moved to the query side (``csrc/attn_latent.hip``): every head's query becomes
+``[U_k^T q_plain | q_rot]``, the attention runs over the cache rows as they lie, and ``U_v`` is applied to each
+head's weighted sum of latents.  A step costs the same whether its keys were cached a step or a thousand steps ago,
+and nothing but c and the rotated part is ever stored.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Sequence
+
+import torch
+
+from .. import ops
+from ..engine.spec import INIT_NORMAL, INIT_ONE_NOISE, MATRIX, VECTOR, TensorSpec
+from .base import Part, StepContext, register_part
+from .linear import Linear
+from .positions import as_rotation
+
+
+class LatentAttentionMixer(Part):
+    def __init__(self, name: str, hidden_size: int, heads: int, dim: int, rot_dim: int, value_dim: int, rank: int,
+                 scale: float, eps: float, positions: Part):
+        """``dim`` / ``rot_dim``: plain and rotated elements of a head's query and key; ``positions`` says how the
+        rotated part turns (a ``Rotation`` over ``rot_dim`` elements)."""
+        self.name, self.hidden_size = name, int(hidden_size)
+        self.heads, self.dim, self.rot_dim, self.value_dim, self.rank = int(heads), int(dim), int(rot_dim), int(value_dim), int(rank)
+        self.scale, self.eps = float(scale), float(eps)
+        self.positions = positions
+        bare = lambda short, i, o: Linear(f"{name}.{short}", i, o, False, weight_name=f"{name}.{short}")
+        self.q = bare("q", hidden_size, self.heads * (self.dim + self.rot_dim))
+        self.down = bare("dkv", hidden_size, self.rank + self.rot_dim)
+        self.out = bare("o", self.heads * self.value_dim, hidden_size)
+        self.q_down: Optional[Linear] = None
+        self.norm_w = self.up_k = self.up_v = None
+
+    @property
+    def cache_row(self) -> int:
+        """Elements the cache holds per token."""
+        return self.rank + self.rot_dim
+
+    def children(self) -> Sequence[Part]:
+        return (self.q, self.down, self.out, self.positions)
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        n = self.name
+        return [TensorSpec(f"{n}.dkv.norm", (self.rank,), VECTOR, INIT_ONE_NOISE),
+                TensorSpec(f"{n}.uk", (self.heads * self.dim, self.rank), MATRIX, INIT_NORMAL),
+                TensorSpec(f"{n}.uv", (self.heads * self.value_dim, self.rank), MATRIX, INIT_NORMAL)]
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        n = self.name
+        self.norm_w, self.up_k, self.up_v = tensors[f"{n}.dkv.norm"], tensors[f"{n}.uk"], tensors[f"{n}.uv"]
+
+    def after_load(self) -> None:
+        self.q_down = Linear.stacked(f"{self.name}.q_dkv", [self.q, self.down])  # both read the layer's input
+
+    def check_sizes(self) -> None:
+        problem = ops.latent_sizes_problem(self.heads, self.dim, self.rot_dim, self.rank)
+        rot = as_rotation(self.positions.rotation())
+        if problem is None and rot is not None:
+            if self.rot_dim == 0:
+                problem = "a rotation needs a rotated part"
+            else:
+                problem = ops.rotation_problem(self.rot_dim, rot.rotary_dim, rot.pairing)
+        if problem is not None:
+            raise ValueError(f"{self.name}: {problem}")
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, call, residual: Optional[torch.Tensor] = None):
+        k_pool, _ = ctx.cache.kv_layer(call.cache_group, call.cache_layer)
+        table = ctx.block_tables[call.cache_group]
+        rot = as_rotation(self.positions.rotation())
+        proj = self.q_down(x)
+        q_full = ops.latent_prep(proj, self.norm_w, self.eps, None if rot is None else rot.inv_freq,
+                                 1.0 if rot is None else rot.scale, None if rot is None else rot.rotary_dim,
+                                 "half" if rot is None else rot.pairing, ctx.token_pos, ctx.token_seq, table, k_pool,
+                                 self.heads, self.dim, self.rot_dim, self.rank, write_cache=call.write_cache)
+        M, D = x.shape[0], self.cache_row
+        # each head's plain query through the transpose of its key expansion: the first `rank` of its frame
+        ops.head_project(proj, self.dim + self.rot_dim, self.up_k, self.heads, self.dim, self.rank, transposed=True,
+                         out=q_full.view(M, self.heads * D), out_head=D)
+        lat = ops.attn_latent(q_full, k_pool, table, ctx.token_seq, ctx.token_pos, self.rank, self.scale)
+        o = ops.head_project(lat.view(M, self.heads * self.rank), self.rank, self.up_v, self.heads, self.rank,
+                             self.value_dim, transposed=False, out_dtype=x.dtype)
+        return self.out(o, add1=residual)
+
+
+register_part("mixer", "latent_attention", LatentAttentionMixer)

@@ -13,7 +13,7 @@ activation and additions.
 """
 from __future__ import annotations
 
-from typing import Dict, List, Optional
+from typing import Dict, List, Optional, Sequence
 
 import torch
 
@@ -23,11 +23,15 @@ from .base import PartialProduct, Part
 
 
 class Linear(Part):
-    def __init__(self, name: str, in_features: int, out_features: int, bias: bool, pieces=None, assemble=None):
+    def __init__(self, name: str, in_features: int, out_features: int, bias: bool, pieces=None, assemble=None,
+                 weight_name: Optional[str] = None, bias_name: Optional[str] = None):
         """``pieces``: (name, rows) of the matrices that a weight file may hold instead of this one (their ``.weight``
         and ``.bias`` under those names), which ``assemble`` (None: one after the other) makes into this one by
-        their rows; the same function is applied to the biases."""
+        their rows; the same function is applied to the biases.  ``weight_name`` / ``bias_name``: the tensors' names
+        in a weight file where they are not ``name + ".weight"`` and ``name + ".bias"``."""
         self.name = name
+        self.weight_name = weight_name or name + ".weight"
+        self.bias_name = bias_name or name + ".bias"
         self.in_features = in_features
         self.out_features = out_features
         self.has_bias = bias
@@ -37,19 +41,36 @@ class Linear(Part):
         self.bias: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> List[TensorSpec]:
-        specs = [TensorSpec(self.name + ".weight", (self.out_features, self.in_features), MATRIX, INIT_NORMAL,
+        specs = [TensorSpec(self.weight_name, (self.out_features, self.in_features), MATRIX, INIT_NORMAL,
                             pieces=tuple((n + ".weight", (rows, self.in_features)) for n, rows in self.pieces),
                             assemble=self.assemble)]
         if self.has_bias:
-            specs.append(TensorSpec(self.name + ".bias", (self.out_features,), VECTOR, INIT_ZERO_NOISE,
+            specs.append(TensorSpec(self.bias_name, (self.out_features,), VECTOR, INIT_ZERO_NOISE,
                                     pieces=tuple((n + ".bias", (rows,)) for n, rows in self.pieces),
                                     assemble=self.assemble))
         return specs
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
-        self.weight = tensors[self.name + ".weight"]
-        self.bias = tensors[self.name + ".bias"] if self.has_bias else None
+        self.weight = tensors[self.weight_name]
+        self.bias = tensors[self.bias_name] if self.has_bias else None
         self.joined = None  # (both matrices as one, the other Linear) after ``join``
+
+    @staticmethod
+    def stacked(name: str, layers: "Sequence[Linear]") -> "Linear":
+        """One layer whose rows are those of ``layers`` (loaded, one input size, no bias applied by it) one after
+        the other, for products of the same input that are to run as one.  The layers' own matrices become views of
+        the stacked one, so nothing is held twice; biases stay with the layers."""
+        ws = [l.weight for l in layers]
+        if any(w is None for w in ws) or len({(w.dtype, w.device, w.shape[1]) for w in ws}) != 1:
+            raise ValueError(f"{name}: layers to stack must be loaded and agree in type, device and input size")
+        both = torch.cat(ws, dim=0).contiguous()
+        out = Linear(name, ws[0].shape[1], both.shape[0], False)
+        out.weight, out.bias, out.joined = both, None, None
+        at = 0
+        for l in layers:
+            l.weight = both[at:at + l.out_features]
+            at += l.out_features
+        return out
 
     @staticmethod
     def join(first: "Linear", second: "Linear") -> bool:
@@ -222,17 +243,18 @@ class PendingProjection:
 class Embedding(Part):
     """``h[t] = E[id_t]``, no scaling (src/transformers/models/falcon/modeling_falcon.py:835, :895-896)."""
 
-    def __init__(self, name: str, vocab_size: int, hidden_size: int):
+    def __init__(self, name: str, vocab_size: int, hidden_size: int, weight_name: Optional[str] = None):
         self.name = name
+        self.weight_name = weight_name or name + ".weight"
         self.vocab_size = vocab_size
         self.hidden_size = hidden_size
         self.weight: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> List[TensorSpec]:
-        return [TensorSpec(self.name + ".weight", (self.vocab_size, self.hidden_size), MATRIX, INIT_NORMAL)]
+        return [TensorSpec(self.weight_name, (self.vocab_size, self.hidden_size), MATRIX, INIT_NORMAL)]
 
     def load(self, tensors) -> None:
-        self.weight = tensors[self.name + ".weight"]
+        self.weight = tensors[self.weight_name]
 
     def forward(self, ids: torch.Tensor) -> torch.Tensor:
         return ops.embed(self.weight, ids)
@@ -243,11 +265,13 @@ class OutputHead(Part):
     (src/transformers/models/falcon/modeling_falcon.py:1163-1168, :1230; the reference casts the
     rows it samples from to 32-bit, src/transformers/generation/utils.py:3247)."""
 
-    def __init__(self, name: str, vocab_size: int, hidden_size: int, tied_to: Optional[str]):
+    def __init__(self, name: str, vocab_size: int, hidden_size: int, tied_to: Optional[str], scale: float = 1.0):
+        """``scale``: a factor on the logits (applied to the 32-bit result)."""
         self.name = name
         self.vocab_size = vocab_size
         self.hidden_size = hidden_size
         self.tied_to = tied_to
+        self.scale = float(scale)
         self.weight: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> List[TensorSpec]:
@@ -258,6 +282,9 @@ class OutputHead(Part):
         self.weight = tensors[self.name + ".weight"]
 
     def forward(self, h: torch.Tensor) -> torch.Tensor:
+        return ops.scale_(self._product(h), self.scale)
+
+    def _product(self, h: torch.Tensor) -> torch.Tensor:
         if h.dtype == torch.float32:
             return ops.gemm_f32(h, self.weight)
         if ops.gemm_skinny_ok(h, self.weight):

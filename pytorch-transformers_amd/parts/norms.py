@@ -63,4 +63,37 @@ class LayerNorm(Part):
         return x, a, m
 
 
+class RMSNorm(Part):
+    """``x / sqrt(mean(x^2) + eps) * (offset + w)`` in 32-bit, eps inside the root.  ``offset`` 1 is for a gain that
+    is stored around zero, 0 for one stored as it is applied.  With ``groups`` > 1 a row is cut into that many equal
+    parts, each divided by its own root mean square.  ``name`` is the weight's name in the file as it stands.
+
+    The input may be 32-bit in a model whose compute type is narrower (a residual stream kept wide); the result
+    comes in the compute type, and on request in 32-bit as well (``apply``)."""
+
+    def __init__(self, name: str, size: int, eps: float, offset: float = 0.0, groups: int = 1):
+        if groups < 1 or size % groups:
+            raise ValueError(f"{name}: {size} features do not split into {groups} equal groups")
+        self.name, self.size, self.eps, self.offset, self.groups = name, int(size), float(eps), float(offset), int(groups)
+        self.weight: Optional[torch.Tensor] = None
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        return [TensorSpec(self.name, (self.size,), VECTOR, INIT_ZERO_NOISE if self.offset else INIT_ONE_NOISE)]
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        self.weight = tensors[self.name]
+
+    def apply(self, x: torch.Tensor, dtype: torch.dtype, **how):
+        """``ops.rmsnorm`` with this norm's weight and constants: ``(narrow, wide)``."""
+        return ops.rmsnorm(x, self.weight, self.eps, dtype, offset=self.offset, groups=self.groups, **how)
+
+    def forward(self, x: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        return self.apply(x, x.dtype, rows=rows)[0]
+
+    def forward_wide(self, x, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """The norm of a ``WideResidual``'s 32-bit side, in its compute type."""
+        return self.apply(x.wide, x.narrow.dtype, rows=rows)[0]
+
+
 register_part("norm", "layernorm", LayerNorm)
+register_part("norm", "rmsnorm", RMSNorm)

@@ -81,8 +81,12 @@ class RotaryPositions(NoPositions):
 
     def __init__(self, head_dim: int, theta: float, scaling_factor: float = 1.0, attention_scaling: float = 1.0,
                  inv_freq: Optional[torch.Tensor] = None, dynamic_factor: Optional[float] = None,
-                 trained_positions: Optional[int] = None):
-        """``inv_freq`` given: a table of ``head_dim / 2`` frequencies of another scheme (``yarn_frequencies``,
+                 trained_positions: Optional[int] = None, rotary_dim: Optional[int] = None, pairing: str = "half"):
+        """``rotary_dim`` (with the default frequencies only): the first so many elements of a head are rotated, with
+        the frequencies ``theta^(-2i / rotary_dim)``, and the rest pass; ``pairing`` ``"interleaved"`` pairs the
+        neighbours (2i, 2i + 1) instead of (i, i + half).
+
+        ``inv_freq`` given: a table of ``head_dim / 2`` frequencies of another scheme (``yarn_frequencies``,
         ``llama3_frequencies``, ``longrope_frequencies``); cosines and sines are multiplied by
         ``attention_scaling`` (src/transformers/models/falcon/modeling_falcon.py:162-166).
 
@@ -108,7 +112,17 @@ class RotaryPositions(NoPositions):
             if self.trained_positions is None or self.trained_positions <= 0 or self.dynamic_factor < 1.0 or head_dim <= 2:
                 raise ValueError("dynamic frequencies need a factor >= 1, the trained context length and a head size "
                                  f"above 2 (factor {dynamic_factor}, context {trained_positions}, head size {head_dim})")
-        if inv_freq is not None:
+        self.rotary_dim = None if rotary_dim is None else int(rotary_dim)
+        self.pairing = pairing
+        if self.rotary_dim is not None:
+            if inv_freq is not None or dynamic_factor is not None:
+                raise ValueError("a rotation of part of a head goes with the default frequencies only")
+            if self.rotary_dim < 2 or self.rotary_dim % 2 or self.rotary_dim > head_dim:
+                raise ValueError(f"rotary_dim must be even, from 2 up to the head size {head_dim}; got {rotary_dim}")
+            inv = default_frequencies(self.rotary_dim, self.theta)
+            if self.scaling_factor != 1.0:
+                inv = inv / self.scaling_factor
+        elif inv_freq is not None:
             if tuple(inv_freq.shape) != (head_dim // 2,):
                 raise ValueError(f"a frequency table for head size {head_dim} has {head_dim // 2} entries, got "
                                  f"{tuple(inv_freq.shape)}")
@@ -123,7 +137,7 @@ class RotaryPositions(NoPositions):
         self.inv_freq = self.inv_freq.to(device)
 
     def rotation(self) -> Rotation:
-        return Rotation(self.inv_freq, self.attention_scaling)
+        return Rotation(self.inv_freq, self.attention_scaling, self.rotary_dim, self.pairing)
 
     def rotation_for(self, ctx) -> Rotation:
         """The rotation for one step: the table, or with dynamic scaling one table per sequence of the step,
@@ -138,7 +152,7 @@ class RotaryPositions(NoPositions):
         if table is None:
             table = ctx.extras[key] = ops.rope_dynamic_table(ctx.seq_start, ctx.cu_tokens, self.head_dim, self.theta,
                                                              self.dynamic_factor, self.trained_positions)
-        return Rotation(table, self.attention_scaling)
+        return Rotation(table, self.attention_scaling, self.rotary_dim, self.pairing)
 
 
 def default_frequencies(head_dim: int, theta: float) -> torch.Tensor:
