@@ -117,7 +117,7 @@ extern "C" int pta_conv_silu(float* out, const void* in, long ld, const float* w
                              int M, int C, int K, int dtype, void* stream) {
     PTA_REQUIRE(M > 0 && n_seqs > 0 && C > 0, "conv_silu: tokens=%d sequences=%d channels=%d must be positive", M, n_seqs, C);
     PTA_REQUIRE(K >= 1 && K <= PTA_CONV_MAX_TAPS, "conv_silu: %d taps are outside 1..%d", K, PTA_CONV_MAX_TAPS);
-    PTA_REQUIRE(out && in && w && tail && cu_tokens && token_seq && seq_slot, "conv_silu: null pointer");
+    PTA_REQUIRE(out && in && w && (tail || K == 1) && cu_tokens && token_seq && seq_slot, "conv_silu: null pointer");
     PTA_REQUIRE(ld >= C && tail_ld >= (long)(K - 1) * C, "conv_silu: rows lie closer together than they are long");
     PTA_REQUIRE(n_seqs <= 65535 && C <= 65535 * 64, "conv_silu: too many sequences or channels for one launch");
     PTA_REQUIRE(dtype == PTA_F32 || dtype == PTA_BF16, "conv_silu: unknown dtype %d", dtype);

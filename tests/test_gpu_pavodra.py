@@ -1,0 +1,447 @@
+"""The Pavodra design on the GPU against the plain implementation (``plain_pavodra``): every mechanism alone, then
+whole models of several shapes through the step function, the cache, captured decode steps and ``generate``.
+
+The tests make their own small configurations and weights.  Sizes are chosen so that nothing is equal that need not
+be (plain, rotated, value and latent sizes of a head; heads and groups; norm groups), and a far key, a page border
+or a stale state shows in the result instead of drowning in averages.
+"""
+import json
+import os
+
+import pytest
+import torch
+
+import helpers
+import plain_pavodra as P
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [("float32", 3e-5), ("bfloat16", 4e-2)]
+TORCH = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+def _rand(*shape, seed=0, scale=1.0):
+    return torch.randn(*shape, generator=torch.Generator().manual_seed(seed)) * scale
+
+
+def _bf16(t):
+    return t.to(torch.bfloat16).double()
+
+
+def _close(got, want, rel, what):
+    got, want = got.double().cpu(), want.double()
+    assert got.shape == want.shape, f"{what}: {tuple(got.shape)} vs {tuple(want.shape)}"
+    assert torch.isfinite(got).all(), f"{what}: not finite"
+    scale = max(1e-6, float(want.abs().max()))
+    err = float((got - want).abs().max())
+    assert err <= rel * scale, f"{what}: max |diff| {err:.3e} > {rel} x {scale:.3e}"
+
+
+# ---- configurations ---------------------------------------------------------------------------------------------
+def attn(heads=3, dim=24, rot_dim=12, vdim=20, rank=40, dims=8, base=10000.0, scale=0.17):
+    return {"type": "latent_attention", "mixer": {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim,
+                                                  "kv_rank": rank, "scale": scale, "rot": {"base": base, "dims": dims}}}
+
+
+def gru(width=72):
+    return {"type": "mingru", "mixer": {"width": width}}
+
+
+def ssm(heads=4, vdim=12, state=10, groups=2, conv=3, norm_groups=3):
+    return {"type": "mamba2", "mixer": {"heads": heads, "vdim": vdim, "state": state, "groups": groups, "conv": conv,
+                                        "norm_groups": norm_groups}}
+
+
+def with_mlp(layer, ff):
+    return dict(layer, mlp=None if ff is None else {"kind": "dense", "ff": ff})
+
+
+def config(layers, vocab=131, width=48, eps=1e-5, mult=0.4, logit_scale=1.5):
+    return {"architecture": "Pavodra", "vocab": vocab, "width": width, "layers": layers, "norm": {"eps": eps},
+            "residual_mult": mult, "logit_scale": logit_scale}
+
+
+CONFIGS = {
+    # every mixer twice with different sizes, a layer without feed-forward, two shapes of latent cache rows
+    "mixed": config([with_mlp(attn(), 96), with_mlp(gru(), 64), with_mlp(ssm(), None), with_mlp(attn(2, 16, 8, 16, 24, 8), 80),
+                     with_mlp(gru(40), 56), with_mlp(ssm(2, 20, 6, 1, 4, 1), 72)]),
+    # one group, one norm group, one head: the values that make indices vanish
+    "ones": config([with_mlp(ssm(1, 16, 4, 1, 2, 1), 32), with_mlp(attn(1, 8, 4, 8, 8, 4), 32), with_mlp(gru(8), None)],
+                   vocab=61, width=16, mult=1.0, logit_scale=1.0),
+    # attention only, wide heads: more than one page of keys matters
+    "attention": config([with_mlp(attn(4, 32, 16, 32, 64, 16, 1e6, 0.11), 64), with_mlp(attn(4, 32, 16, 32, 64, 16, 1e6, 0.11), 64)],
+                        vocab=97, width=64),
+}
+
+
+def make_weights(cfg, seed, std=0.25):
+    """Random weights by the design's tensor names, rounded to bfloat16 (so that both compute types hold the same
+    numbers), as float64.  Lively enough that layers matter: gains around one, decays of every size."""
+    from pytorch_transformers_amd.config import AutoConfig
+    from pytorch_transformers_amd.config.registry import lookup
+
+    c = AutoConfig.from_dict(cfg)
+    specs = lookup(c.model_type)[1](c).tensor_specs()
+    g = torch.Generator().manual_seed(seed)
+    w = {}
+    for s in specs:
+        if s.tied_to is not None:
+            continue
+        n = s.name
+        t = torch.randn(s.shape, generator=g)
+        if n.endswith((".norm1", ".norm2")) or n == "final.norm":
+            t = 0.3 * t  # stored around zero
+        elif n.endswith(".norm"):
+            t = 1.0 + 0.3 * t
+        elif n.endswith(".dwa"):
+            t = 0.3 * t
+            t[-1] += 1.0
+        elif n.endswith(".A_log"):
+            t = t  # decays exp(-exp(N(0,1)) dt)
+        elif n.endswith((".dt_bias", ".D", ".b")):
+            t = 0.5 * t
+        elif n.endswith(".conv"):
+            t = 0.5 * t
+        elif n == "embed":
+            t = t
+        else:
+            t = t * std * (48.0 / s.shape[-1]) ** 0.5
+        w[n] = _bf16(t)
+    return w
+
+
+def write_model(folder, cfg, w):
+    from safetensors.torch import save_file
+
+    os.makedirs(folder, exist_ok=True)
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    save_file({k: v.to(torch.bfloat16).contiguous() for k, v in w.items()}, os.path.join(folder, "model.safetensors"),
+              metadata={"format": "pt"})
+    return str(folder)
+
+
+def load(folder, dtype):
+    from pytorch_transformers_amd import AutoModelForCausalLM
+
+    return AutoModelForCausalLM.from_pretrained(str(folder), dtype=dtype)
+
+
+def plain_all(cfg, w, reqs):
+    return {rid: P.forward(cfg, w, toks)[0].float() for rid, toks in reqs.items()}
+
+
+# ---- the kernels alone ---------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype,rel", DTYPES)
+def test_rms_norm_with_gate_groups_rows_and_residual(dtype, rel):
+    from pytorch_transformers_amd import ops
+
+    dt = TORCH[dtype]
+    for M, H, groups in ((5, 48, 1), (3, 90, 3), (70, 2304, 2), (2, 7, 7)):
+        x, gate, res = _bf16(_rand(M, H, seed=1, scale=2.0)), _bf16(_rand(M, H, seed=2)), _rand(M, H, seed=3).double()
+        w = _bf16(_rand(H, seed=4, scale=0.3))
+        plain = P.rms(x.view(M, groups, H // groups), 1e-3).reshape(M, H) * (1.0 + w)
+        wd, xd = w.float().cuda(), x.to(dt).cuda()
+        narrow, wide = ops.rmsnorm(xd, wd, 1e-3, dt, offset=1.0, groups=groups, want_wide=True)
+        _close(wide, plain, 3e-6, f"rms {M}x{H}/{groups} wide")
+        _close(narrow, plain, rel, f"rms {M}x{H}/{groups} narrow")
+        assert narrow.dtype == dt and wide.dtype == torch.float32
+        # a gate in front, a plain gain, the input in 32-bit, the result added to a residual times a constant
+        gated = x * P.silu(gate)
+        plain = res + 0.3 * P.rms(gated.view(M, groups, H // groups), 1e-3).reshape(M, H) * w
+        wide = ops.rmsnorm(x.float().cuda(), wd, 1e-3, dt, groups=groups, gate=gate.to(dt).cuda(),
+                           residual=res.float().cuda(), mult=0.3, want_wide=True, want_narrow=False)[1]
+        _close(wide, plain, 3e-6, f"gated rms {M}x{H}/{groups}")
+        # rows picked out of a wider matrix
+        rows = torch.tensor([M - 1, 0], dtype=torch.int32).cuda()
+        other = _bf16(x + 1.0)
+        both = torch.cat([x, other], 1).to(dt).cuda()
+        got = ops.rmsnorm(both[:, H:], wd, 1e-3, dt, offset=1.0, rows=rows)[0]
+        _close(got, (P.rms(other, 1e-3) * (1.0 + w))[[M - 1, 0]], rel, f"rms rows {M}x{H}")
+
+
+@pytest.mark.parametrize("dtype,rel", DTYPES)
+def test_depth_mix_adds_the_streams_in_order(dtype, rel):
+    from pytorch_transformers_amd import ops
+
+    for M, H, count, total in ((3, 10, 2, 4), (9, 64, 5, 5), (1, 7, 3, 6)):
+        planes = _rand(total, M, H, seed=5).double()
+        coef = _rand(count, seed=6).double()
+        want = sum(coef[j] * planes[j] for j in range(count))
+        narrow, wide = ops.depth_mix(planes.float().cuda(), coef.float().cuda(), count, TORCH[dtype])
+        _close(wide, want, 3e-6, "depth mix wide")
+        _close(narrow, want, rel, "depth mix narrow")
+
+
+def _ctx(cache, slots, new_tokens, dtype):
+    import numpy as np
+
+    from pytorch_transformers_amd.engine.step import plan_step
+    from pytorch_transformers_amd.parts.base import StepContext
+
+    plan = plan_step(cache, slots, [[0] * n for n in new_tokens], "all", 10)
+    i32 = lambda a: torch.as_tensor(np.asarray(a), dtype=torch.int32).cuda()
+    ctx = StepContext(dtype=dtype, device=torch.device("cuda:0"), n_seqs=plan.n_seqs, n_tokens=plan.n_tokens,
+                      token_seq=i32(plan.token_seq), token_pos=i32(plan.token_pos), cu_tokens=i32(plan.cu_tokens),
+                      seq_start=i32(plan.starts), seq_slot=i32(plan.slots),
+                      block_tables={g: i32(t) for g, t in plan.block_tables.items()}, cache=cache, slots=plan.slots,
+                      new_tokens=plan.new_tokens, starts=plan.starts, is_decode=plan.is_decode, max_len=plan.max_len)
+    return ctx, plan
+
+
+def _run_mixer(mixer, group, dtype, inputs, cuts_per_seq):
+    """Feed each sequence of ``inputs`` (float64 ``[T, hidden]``) through ``mixer`` in the given cuts, all sequences
+    of a round in one step; returns the outputs per sequence."""
+    from pytorch_transformers_amd.cache.paged import PagedCache
+    from pytorch_transformers_amd.engine.spec import LayerCall
+
+    cache = PagedCache([group], 4096, dtype, "cuda:0", max_slots=8)
+    call = LayerCall(0, group.name, 0)
+    slots = [cache.alloc() for _ in inputs]
+    at = [0] * len(inputs)
+    outs = [[] for _ in inputs]
+    rounds = max(len(c) for c in cuts_per_seq)
+    for r in range(rounds):
+        live = [i for i, c in enumerate(cuts_per_seq) if r < len(c)]
+        ns = [cuts_per_seq[i][r] for i in live]
+        ctx, plan = _ctx(cache, [slots[i] for i in live], ns, dtype)
+        x = torch.cat([inputs[i][at[i]:at[i] + n] for i, n in zip(live, ns)]).to(dtype).cuda()
+        y = mixer.forward(x, ctx, call)
+        cache.commit(plan.slots, plan.new_tokens)
+        o = 0
+        for i, n in zip(live, ns):
+            outs[i].append(y[o:o + n].double().cpu())
+            at[i] += n
+            o += n
+    return [torch.cat(o) for o in outs]
+
+
+def _load_part(part, w, dtype):
+    from pytorch_transformers_amd.weights.loader import device_dtype_for
+
+    part.load_all({s.name: w[s.name].to(device_dtype_for(s, dtype)).cuda() for s in part.all_tensor_specs()})
+    if hasattr(part, "after_load"):
+        part.after_load()
+
+    def walk(p):
+        if hasattr(p, "to"):
+            p.to("cuda:0")
+        for c in p.children():
+            walk(c)
+
+    walk(part)
+
+
+def _part_weights(part, seed, std=0.3):
+    g = torch.Generator().manual_seed(seed)
+    w = {}
+    for s in part.all_tensor_specs():
+        t = torch.randn(s.shape, generator=g)
+        t = 1.0 + 0.3 * t if s.name.endswith(".norm") else t * (0.5 if len(s.shape) == 1 or s.name.endswith(".conv") else std)
+        w[s.name] = _bf16(t)
+    return w
+
+
+CUTS = [[61], [1] * 9 + [2, 50], [30, 2, 2, 27], [64 - 3, ]]  # whole; token by token, then a rest; portions down to two
+
+
+@pytest.mark.parametrize("dtype,rel", DTYPES)
+def test_gated_scan_mixer_alone(dtype, rel):
+    from pytorch_transformers_amd.engine.spec import CACHE_STATE, CacheGroupSpec
+    from pytorch_transformers_amd.parts import GatedScanMixer
+
+    dt = TORCH[dtype]
+    for hidden, width in ((24, 40), (16, 1), (8, 130)):
+        mixer = GatedScanMixer("m", hidden, width)
+        w = _part_weights(mixer, 3)
+        _load_part(mixer, w, dt)
+        group = CacheGroupSpec("s", CACHE_STATE, 1, state_shape=mixer.state_shape)
+        inputs = [_bf16(_rand(sum(c), hidden, seed=10 + i, scale=2.0)) for i, c in enumerate(CUTS)]
+        got = _run_mixer(mixer, group, dt, inputs, CUTS)
+        for i, h in enumerate(inputs):
+            want = P.mingru(h, {k.replace("m.", "l.mix."): v for k, v in w.items()}, "l")[0]
+            _close(got[i], want, rel, f"gated scan {hidden}->{width} {dtype} sequence {i}")
+
+
+@pytest.mark.parametrize("dtype,rel", DTYPES)
+def test_state_space_mixer_alone(dtype, rel):
+    from pytorch_transformers_amd.engine.spec import CACHE_STATE, CacheGroupSpec
+    from pytorch_transformers_amd.parts import StateSpaceMixer
+
+    dt = TORCH[dtype]
+    for hidden, m in ((24, ssm()["mixer"]), (16, ssm(1, 70, 5, 1, 1, 2)["mixer"]), (16, ssm(6, 8, 33, 3, 5, 1)["mixer"])):
+        mixer = StateSpaceMixer("m", hidden, m["heads"], m["vdim"], m["state"], m["groups"], m["conv"], m["norm_groups"], 1e-5)
+        w = _part_weights(mixer, 4)
+        _load_part(mixer, w, dt)
+        group = CacheGroupSpec("s", CACHE_STATE, 1, state_shape=mixer.state_shape)
+        inputs = [_bf16(_rand(sum(c), hidden, seed=20 + i, scale=1.5)) for i, c in enumerate(CUTS)]
+        got = _run_mixer(mixer, group, dt, inputs, CUTS)
+        for i, h in enumerate(inputs):
+            want = P.mamba2(h, {k.replace("m.", "l.mix."): v for k, v in w.items()}, "l", m, 1e-5)[0]
+            # (in bfloat16 the rounded input product alone moves this layer by a few percent: see REL_BF16_MODEL)
+            _close(got[i], want, max(rel, 2 * rel if dtype == "bfloat16" else rel), f"state space {m} {dtype} sequence {i}")
+
+
+def _latent_mixer(hidden, m):
+    from pytorch_transformers_amd.parts import LatentAttentionMixer, RotaryPositions
+
+    pos = RotaryPositions(m["rot_dim"], m["rot"]["base"], rotary_dim=m["rot"]["dims"], pairing="interleaved")
+    return LatentAttentionMixer("m", hidden, m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"], m["scale"], 1e-5, pos)
+
+
+@pytest.mark.parametrize("dtype,rel", DTYPES)
+def test_latent_attention_mixer_alone(dtype, rel):
+    from pytorch_transformers_amd.engine.spec import CACHE_FULL, CacheGroupSpec
+
+    dt = TORCH[dtype]
+    cuts = [[150], [60, 3, 1, 1, 2, 63, 20], [64, 64, 1, 21], [127, 1, 1, 21]]  # page borders inside and between steps
+    for hidden, m in ((24, attn()["mixer"]), (16, attn(5, 8, 16, 4, 70, 16, 100.0, 0.3)["mixer"])):
+        mixer = _latent_mixer(hidden, m)
+        w = _part_weights(mixer, 5)
+        _load_part(mixer, w, dt)
+        group = CacheGroupSpec("kv", CACHE_FULL, 1, 1, mixer.cache_row, values=False)
+        inputs = [_bf16(_rand(150, hidden, seed=30 + i, scale=1.5)) for i in range(len(cuts))]
+        got = _run_mixer(mixer, group, dt, inputs, cuts)
+        for i, h in enumerate(inputs):
+            want = P.latent_attention(h, {k.replace("m.", "l.mix."): v for k, v in w.items()}, "l", m, 1e-5)
+            _close(got[i], want, rel, f"latent attention {m} {dtype} sequence {i}")
+
+
+@pytest.mark.parametrize("dtype,rel", DTYPES)
+@pytest.mark.parametrize("far", [0, 3, 63, 64, 127, 128, 500])
+def test_latent_attention_finds_one_far_key(dtype, rel, far):
+    """One key among several hundred is made to stand out: its input is scaled, which scales its rotated key part
+    (the part that no norm flattens), and the query's input is scaled so that the softmax is sharp.  The heads whose
+    query agrees with that key then copy its value, the others shut it out: either way the result hangs on that one
+    cache row, at the sequence's start, on either side of a page border, or far back, in a prompt and in decoding."""
+    from pytorch_transformers_amd.engine.spec import CACHE_FULL, CacheGroupSpec
+
+    dt = TORCH[dtype]
+    m = attn(4, 16, 16, 12, 24, 8, 10000.0, 0.25)["mixer"]
+    mixer = _latent_mixer(32, m)
+    w = _part_weights(mixer, 6)
+    _load_part(mixer, w, dt)
+    group = CacheGroupSpec("kv", CACHE_FULL, 1, 1, mixer.cache_row, values=False)
+    T = 640
+    h = _rand(T, 32, seed=40, scale=0.3)
+    h[far] *= 40.0
+    h[-1] *= 6.0
+    h[-2] *= 6.0
+    h = _bf16(h)
+    pw = {k.replace("m.", "l.mix."): v for k, v in w.items()}
+    want = P.latent_attention(h, pw, "l", m, 1e-5)
+    quiet = h.clone()
+    quiet[far] = h[far] / 40.0
+    moved = (P.latent_attention(quiet, pw, "l", m, 1e-5)[-2:] - want[-2:]).abs().max() / want[-2:].abs().max()
+    assert moved > 0.2, "the test's far key does not matter enough to show a fault"
+    got = _run_mixer(mixer, group, dt, [h, h], [[T], [T - 2, 1, 1]])
+    _close(got[0][-2:], want[-2:], rel, f"far key {far} in a prompt")
+    _close(got[1][-2:], want[-2:], rel, f"far key {far} decoded")
+
+
+# ---- whole models ---------------------------------------------------------------------------------------------
+# The 32-bit runs are the sharp ones.  In bfloat16 the weights above (gains around one, decays of every size, norm
+# groups of sixteen elements) make rounding loud: rounding nothing but a state-space layer's input product to
+# bfloat16, in the plain implementation itself, moves that layer's output by 1 % on average and 2.6 % at single
+# tokens, and six layers stand on each other.  So whole models in bfloat16 are held to a tenth of the largest logit;
+# each mechanism alone is held to the usual 4 %.
+REL_BF16_MODEL = 0.1
+
+
+@pytest.mark.parametrize("dtype,rel", [("float32", helpers.REL_F32), ("bfloat16", REL_BF16_MODEL)])
+@pytest.mark.parametrize("name", sorted(CONFIGS))
+def test_schedules_give_the_plain_logits(tmp_path, name, dtype, rel):
+    """Whole prompts, prompt then token by token, unequal batches decoded together, requests that join and leave
+    with prompts in portions down to one token: all the plain logits, with slots and pages freed and used again."""
+    from pytorch_transformers_amd.engine.replay import Replayer
+
+    cfg = CONFIGS[name]
+    w = make_weights(cfg, seed=11)
+    model = load(write_model(tmp_path / name, cfg, w), dtype)
+    reqs = helpers.make_requests(cfg["vocab"], [9, 70, 131, 1, 64, 65, 2], seed=3)
+    want = plain_all(cfg, w, reqs)
+    rp = Replayer(model, 1024, max_slots=8)
+    for label, records in (("whole", helpers.schedule_whole(reqs)), ("tail", helpers.schedule_tail(reqs, 40)),
+                           ("batches", helpers.schedule_batches(reqs, 3)),
+                           ("staggered", helpers.schedule_staggered(reqs, chunks=(None, 2, 19, 1))),
+                           ("batches again", helpers.schedule_batches(reqs, 4, decode=(1, 30, 2, 5)))):
+        got = helpers.run_schedule(rp, records)
+        for rid in reqs:
+            helpers.assert_close(got[rid], want[rid], rel, f"{name} {dtype} {label} {rid}")
+        assert not rp.cache.live_slots()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_captured_decode_steps_equal_direct_ones(tmp_path, dtype):
+    """Decode steps replayed from a captured graph give the bits of the same steps launched one by one, with batches
+    that are padded to the captured size (the padding rows move the scratch slot's state, never a sequence's)."""
+    from pytorch_transformers_amd.engine.replay import Replayer
+
+    cfg = CONFIGS["mixed"]
+    folder = write_model(tmp_path / "m", cfg, make_weights(cfg, seed=12))
+    reqs = helpers.make_requests(cfg["vocab"], [9, 30, 70, 3, 41, 12, 25, 8, 19, 33, 50], seed=4)
+    records = helpers.schedule_batches(reqs, 3, decode=(5, 2, 8)) + \
+        [dict(r, step=r["step"] + 1000) for r in helpers.schedule_batches(reqs, 11, decode=(2, 9, 4))]
+    outs = {}
+    for graphs in (False, True):
+        model = load(folder, dtype)
+        assert model.use_graphs
+        model.use_graphs = graphs
+        rp = Replayer(model, 2048, max_slots=16)
+        outs[graphs] = [rp.run(rec) for rec in records]
+        torch.cuda.synchronize()
+    for rec, a, b in zip(records, outs[False], outs[True]):
+        assert (a is None) == (b is None)
+        if a is not None:
+            assert torch.equal(a, b), f"step {rec['step']}: a captured step differs from the same step launched directly"
+
+
+@pytest.mark.parametrize("dtype,rel", [("float32", helpers.REL_F32), ("bfloat16", REL_BF16_MODEL)])
+def test_long_decoding_and_a_loud_far_token(tmp_path, dtype, rel):
+    """300 tokens decoded one by one after a short prompt (states and pages carried over hundreds of steps), with a
+    token near the start whose embedding is loud, so that the first layer's attention keeps looking back at it."""
+    from pytorch_transformers_amd.engine.replay import Replayer
+
+    cfg = CONFIGS["mixed"]
+    w = make_weights(cfg, seed=13)
+    w["embed"][7] = _bf16(w["embed"][7] * 12.0)
+    model = load(write_model(tmp_path / "m", cfg, w), dtype)
+    toks = [t if t != 7 else 8 for t in helpers.make_requests(cfg["vocab"], [330], seed=5)["r0"]]
+    toks[2] = 7
+    reqs = {"long": toks}
+    want = plain_all(cfg, w, reqs)
+    got = helpers.run_schedule(Replayer(model, 1024, max_slots=2), helpers.schedule_tail(reqs, 300))
+    helpers.assert_close(got["long"], want["long"], rel, f"long decoding {dtype}")
+
+
+def test_greedy_generation_follows_the_plain_model(tmp_path):
+    cfg = CONFIGS["mixed"]
+    w = make_weights(cfg, seed=14)
+    model = load(write_model(tmp_path / "m", cfg, w), "float32")
+    reqs = helpers.make_requests(cfg["vocab"], [5, 17, 2], seed=6)
+    out = model.generate(list(reqs.values()), max_new_tokens=12, do_sample=False, eos_token_id=None)
+    for seq, toks in zip(out, reqs.values()):
+        toks = list(toks)
+        for _ in range(12):
+            toks.append(int(P.forward(cfg, w, toks)[0][-1].argmax()))
+        assert list(seq) == toks
+
+
+def test_random_weights_from_a_configuration_run(tmp_path):
+    """The framework's own random-weights mode writes the design's tensor names, and what it writes loads and steps."""
+    from safetensors import safe_open
+
+    from pytorch_transformers_amd import AutoModelForCausalLM
+    from pytorch_transformers_amd.config import AutoConfig
+    from pytorch_transformers_amd.weights import write_random_model
+
+    cfg = AutoConfig.from_dict(CONFIGS["ones"])
+    folder = write_random_model(str(tmp_path / "r"), cfg, seed=1, std=0.1)
+    with safe_open(os.path.join(folder, "model.safetensors"), framework="pt") as f:
+        names = set(f.keys())
+    assert {"embed", "final.norm", "l0.mix.in", "l0.mix.conv.b", "l1.mix.dkv.norm", "l2.mix.z.b", "l2.dwa"} <= names
+    assert "l2.mlp.up" not in names and "l2.norm2" not in names  # the layer without a feed-forward
+    model = AutoModelForCausalLM.from_pretrained(folder, dtype="bfloat16")
+    cache = model.new_cache(256)
+    logits = model.step(cache, [cache.alloc()], [[1, 2, 3]], "all")
+    assert logits.shape == (3, cfg.vocab) and torch.isfinite(logits).all()
