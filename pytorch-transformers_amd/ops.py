@@ -1247,11 +1247,30 @@ def head_project(x: torch.Tensor, x_head: int, w: torch.Tensor, heads: int, K: i
     return out
 
 
+LATENT_MFMA = os.environ.get("PTA_LATENT_MFMA", "1") != "0"
+LATENT_SPLIT_WORKGROUPS = 1024  # a decode launch cuts its keys into ranges until it has about so many workgroups
+
+
+def attn_latent_mfma_ok(k_pool: torch.Tensor, rank: int) -> bool:
+    """Whether the matrix-core kernel takes this cache (bfloat16, a size class built for its rows)."""
+    return (LATENT_MFMA and k_pool.dtype == torch.bfloat16
+            and bool(load_library().pta_attn_latent_mfma_ok(int(rank), int(k_pool.shape[-1]))))
+
+
+def latent_decode_split(n_seqs: int, heads: int, max_len: int):
+    """(keys per range, ranges) of a decode launch: ranges of a multiple of 64 keys, enough of them to fill the chip."""
+    tiles = (heads + 63) // 64
+    want = max(1, min((max_len + 63) // 64, LATENT_SPLIT_WORKGROUPS // max(1, n_seqs * tiles)))
+    size = ((max_len + want - 1) // want + 63) // 64 * 64
+    return size, (max_len + size - 1) // size
+
+
 def attn_latent(q_full: torch.Tensor, k_pool: torch.Tensor, block_table, token_seq, token_pos, rank: int,
-                scale: float) -> torch.Tensor:
+                scale: float, ctx=None) -> torch.Tensor:
     """Causal attention of every token over its sequence's cache rows ``[rank + rot_dim]``, whose first ``rank``
     elements are also the values: ``q_full`` ``[tokens, heads, rank + rot_dim]`` (32-bit) -> ``[tokens, heads,
-    rank]`` (32-bit)."""
+    rank]`` (32-bit).  With the step's context (``ctx``) and a bfloat16 cache of a size that is built, the kernel on
+    the matrix cores runs, its keys cut into ranges when every sequence brings one token; else the 32-bit kernel."""
     _need(q_full, "q_full", torch.float32)
     M, H, D = q_full.shape
     if k_pool.dim() != 4 or tuple(k_pool.shape[1:]) != (1, 64, D) or not k_pool.is_cuda or not k_pool.is_contiguous():
@@ -1260,8 +1279,23 @@ def attn_latent(q_full: torch.Tensor, k_pool: torch.Tensor, block_table, token_s
     _need(token_seq, "token_seq", torch.int32, (M,))
     _need(token_pos, "token_pos", torch.int32, (M,))
     out = torch.empty((M, H, rank), dtype=torch.float32, device=q_full.device)
-    if M:
-        _call("pta_attn_latent", _ptr(out), _ptr(q_full), _ptr(k_pool), _ptr(block_table), block_table.shape[1],
-              _ptr(token_seq), _ptr(token_pos), M, H, int(rank), D - int(rank), ctypes.c_float(scale),
-              dtype_code(k_pool.dtype), _stream())
+    if M == 0:
+        return out
+    if ctx is not None and attn_latent_mfma_ok(k_pool, rank):
+        n = block_table.shape[0]
+        _need(ctx.cu_tokens, "cu_tokens", torch.int32, (n + 1,))
+        _need(ctx.seq_start, "seq_start", torch.int32, (n,))
+        size, splits = latent_decode_split(n, H, ctx.max_len) if ctx.is_decode else (0, 1)
+        po = pm = pl = None
+        if splits > 1:
+            po = torch.empty((M, H, splits, rank), dtype=torch.float32, device=q_full.device)
+            pm = torch.empty((M, H, splits), dtype=torch.float32, device=q_full.device)
+            pl = torch.empty((M, H, splits), dtype=torch.float32, device=q_full.device)
+        _call("pta_attn_latent_mfma", _ptr(out), _ptr(po), _ptr(pm), _ptr(pl), _ptr(q_full), _ptr(k_pool), _ptr(block_table),
+              block_table.shape[1], _ptr(ctx.cu_tokens), _ptr(ctx.seq_start), n, int(max(ctx.new_tokens)), M, H, int(rank),
+              D - int(rank), ctypes.c_float(scale), int(size), int(splits), _stream())
+        return out
+    _call("pta_attn_latent", _ptr(out), _ptr(q_full), _ptr(k_pool), _ptr(block_table), block_table.shape[1],
+          _ptr(token_seq), _ptr(token_pos), M, H, int(rank), D - int(rank), ctypes.c_float(scale),
+          dtype_code(k_pool.dtype), _stream())
     return out

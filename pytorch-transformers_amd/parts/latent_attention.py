@@ -82,7 +82,7 @@ class LatentAttentionMixer(Part):
         # each head's plain query through the transpose of its key expansion: the first `rank` of its frame
         ops.head_project(proj, self.dim + self.rot_dim, self.up_k, self.heads, self.dim, self.rank, transposed=True,
                          out=q_full.view(M, self.heads * D), out_head=D)
-        lat = ops.attn_latent(q_full, k_pool, table, ctx.token_seq, ctx.token_pos, self.rank, self.scale)
+        lat = ops.attn_latent(q_full, k_pool, table, ctx.token_seq, ctx.token_pos, self.rank, self.scale, ctx=ctx)
         o = ops.head_project(lat.view(M, self.heads * self.rank), self.rank, self.up_v, self.heads, self.rank,
                              self.value_dim, transposed=False, out_dtype=x.dtype)
         return self.out(o, add1=residual)
