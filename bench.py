@@ -357,8 +357,122 @@ def extra_points(sizes, limit, dtype):
     return {f"{tag}_{k}": v for k, v in json.loads(lines[-1]).items()}
 
 
+# ---- the Pavodra design beside the closest Falcon model at equal layer sizes (--design pavodra) ---------------------
+PAVODRA_SIZES = {
+    # width, feed-forward, heads of the latent attention (128 plain + 64 rotated elements, values of 128, latents of 512),
+    # heads of the state-space layers (64 elements each, 128 state rows, 8 groups)
+    "2k": dict(width=2048, ff=8192, heads=16, ssm_heads=64),
+    "4k": dict(width=4096, ff=16384, heads=32, ssm_heads=128),
+}
+PAVODRA_KERNEL_LABELS = {
+    "pta_rmsnorm": "RMS norm (+ gate, + residual into the 32-bit stream)",
+    "pta_depth_mix": "weighted sum of the layers' streams",
+    "pta_gated_scan": "gated recurrence",
+    "pta_conv_silu": "short convolution + silu (+ its tail)",
+    "pta_ssm_scan": "state-space recurrence",
+    "pta_latent_prep": "latent norm, rotation, cache write",
+    "pta_head_project": "per-head products with the key / value expansions",
+    "pta_attn_latent_mfma": "attention over the latent cache (+ merge of key ranges)",
+    "pta_attn_latent": "attention over the latent cache, 32-bit kernel",
+}
+
+
+def pavodra_config(size, layers, vocab=32768):
+    from pytorch_transformers_amd import PavodraConfig
+
+    z = PAVODRA_SIZES[size]
+    mlp = {"kind": "dense", "ff": z["ff"]}
+    kinds = [
+        {"type": "latent_attention", "mixer": {"heads": z["heads"], "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 512,
+                                               "scale": 192 ** -0.5, "rot": {"base": 10000.0, "dims": 64}}, "mlp": mlp},
+        {"type": "mingru", "mixer": {"width": z["width"]}, "mlp": mlp},
+        {"type": "mamba2", "mixer": {"heads": z["ssm_heads"], "vdim": 64, "state": 128, "groups": 8, "conv": 4,
+                                     "norm_groups": 8}, "mlp": mlp},
+    ]
+    return PavodraConfig(vocab=vocab, width=z["width"], layers=[kinds[i % 3] for i in range(layers)], norm={"eps": 1e-6},
+                         residual_mult=0.3, logit_scale=1.0, initializer_range=0.02)
+
+
+def falcon_like(size, layers, vocab=32768):
+    """The closest model the library had: Falcon's new architecture at the same width, feed-forward, depth and
+    vocabulary, heads of 128 in 8 groups."""
+    from pytorch_transformers_amd import FalconConfig
+
+    z = PAVODRA_SIZES[size]
+    return FalconConfig(vocab_size=vocab, hidden_size=z["width"], num_hidden_layers=layers, num_attention_heads=z["width"] // 128,
+                        num_kv_heads=8, new_decoder_architecture=True, num_ln_in_parallel_attn=1, parallel_attn=True,
+                        bias=False, alibi=False, ffn_hidden_size=z["ff"], rope_theta=10000.0, layer_norm_epsilon=1e-5,
+                        max_position_embeddings=8192, tie_word_embeddings=True)
+
+
+def design_record(args):
+    """Prefill and decode throughput of Pavodra models and of Falcon models of the same layer sizes, and the launches of
+    one decode step and one prefill of each with their rates against the published peaks."""
+    import torch
+
+    from pytorch_transformers_amd import AutoModelForCausalLM, GenerationConfig, ops
+    from pytorch_transformers_amd.sampling import Sampler
+
+    ops.load_library()
+    KERNEL_LABELS.update(PAVODRA_KERNEL_LABELS)
+    gen_cfg = GenerationConfig(do_sample=False, eos_token_id=None)
+    layers, T, ctx_len = args.layers or 6, args.prefill_tokens, args.prompt_len
+    out = {"design": "pavodra", "beside": "falcon (new architecture, 8 KV groups of head size 128)", "dtype": args.dtype,
+           "layers": layers, "prefill_tokens": T, "decode_context": ctx_len, "data": "synthetic token ids, random weights",
+           "sizes": {}}
+    dtype = "bfloat16" if args.dtype == "bf16" else "float32"
+    for size in args.design_sizes.split(","):
+        rec = {}
+        for name, cfg in (("pavodra", pavodra_config(size, layers)), ("falcon", falcon_like(size, layers))):
+            model = AutoModelForCausalLM.from_config(cfg, seed=0, dtype=dtype, device="cuda:0")
+            r = {}
+            pt = run_prefill(model, T)
+            r["prefill_tokens_per_s"], r["prefill_ms"] = round(T / pt, 1), round(pt * 1e3, 3)
+            for b in (1, 8, 64):
+                d, _, med = run_decode(model, Sampler, gen_cfg, b, ctx_len, 32, 8, per_step=True)
+                r[f"decode_b{b}_tokens_per_s"], r[f"decode_b{b}_ms_per_step"] = round(b * 32 / d, 1), round(med, 4)
+            if args.dtype == "bf16" and not args.no_points:
+                g = torch.Generator().manual_seed(3)
+                page = model.page_size
+                b = 8
+                prompts = torch.randint(0, model.vocab_size, (b, ctx_len), generator=g).tolist()
+                cache = model.new_cache(b * ((ctx_len + 8 + page - 1) // page * page), max_slots=b)
+                slots = [cache.alloc() for _ in range(b)]
+                model.step(cache, slots, prompts, "last")
+                if name == "pavodra":
+                    row, heads, rank = 576, PAVODRA_SIZES[size]["heads"], 512
+                    kv, fl = b * (ctx_len + 1) * row * 2, 2.0 * heads * (row + rank) * T * (T + 1) / 2
+                else:
+                    kv = b * (ctx_len + 1) * 2 * cfg.kv_heads * cfg.head_dim * 2
+                    fl = 2.0 * cfg.head_dim * cfg.num_attention_heads * T * (T + 1)
+                r["kernels_decode_b8"] = kernel_figures(model, ops, args.dtype, lambda: model.step(cache, slots, [[1]] * b, "last"),
+                                                        attn_bytes=kv)
+                for s_ in slots:
+                    cache.free(s_)
+                del cache
+                prompt = torch.randint(0, model.vocab_size, (T,), generator=g).tolist()
+                cache = model.new_cache((T + page - 1) // page * page * 2, max_slots=2)
+
+                def step():
+                    slot = cache.alloc()
+                    model.step(cache, [slot], [prompt], "last")
+                    cache.free(slot)
+
+                r[f"kernels_prefill_{T}"] = kernel_figures(model, ops, args.dtype, step, attn_flops=fl)
+                del cache
+            rec[name] = r
+            del model
+            torch.cuda.empty_cache()
+        out["sizes"][size] = rec
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
+    ap.add_argument("--design", default=None, choices=["pavodra"],
+                    help="measure that design beside the closest Falcon model at equal layer sizes and print that record "
+                         "instead of the default run's (--layers, --prefill-tokens, --prompt-len and --dtype apply)")
+    ap.add_argument("--design-sizes", default="2k,4k", help="with --design: which of the layer sizes 2k, 4k")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=128)
     ap.add_argument("--warmup", type=int, default=16)
@@ -384,6 +498,10 @@ def main():
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
+
+    if args.design:
+        print(json.dumps(design_record(args)))
+        return 0
 
     import torch
 

@@ -86,17 +86,21 @@ extern "C" int pta_latent_prep(float* q_full, void* k_pool, const void* proj, lo
     return pta_check_launch("latent_prep");
 }
 
-// A small product per head: out[t, h, o] = sum_k in[t, h, k] * W[h][o, k], with W's element (o, k) of head h at
-// w[h * w_head + o * w_o + k * w_k] (so the same launch takes a head's matrix either way round).
-// A workgroup owns (16 tokens, head, 64 outputs); K is walked in pieces of 128 that lie in LDS.
+// A small product per head: out[t, h, o] = sum_k in[t, h, k] * W[h][k, o], with head h's matrix at w + h * K * O,
+// K-major (its rows are inputs), so that neighbouring threads read neighbouring outputs.
+// A workgroup owns (16 tokens, head, 64 outputs); its four waves take a quarter of K each and add up in LDS in wave
+// order.  K is walked in pieces of 128 that lie in LDS.  For steps of few tokens; prompts in bfloat16 go to the
+// vendor library's batched product instead.
 template <typename TI, typename TW, typename TO>
 __global__ __launch_bounds__(256) void head_project_kernel(TO* __restrict__ out, long out_ld, long out_head,
                                                            const TI* __restrict__ in, long in_ld, long in_head,
-                                                           const TW* __restrict__ w, long w_head, long w_o, long w_k,
-                                                           int M, int K, int O) {
+                                                           const TW* __restrict__ w, int M, int K, int O) {
     __shared__ float in_s[16][128 + 1];
-    const int h = blockIdx.y, m0 = blockIdx.z * 16, o = blockIdx.x * 64 + (threadIdx.x & 63), tg = threadIdx.x >> 6;
-    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    __shared__ float part[3][16][64];
+    const int h = blockIdx.y, m0 = blockIdx.z * 16, lane = threadIdx.x & 63, o = blockIdx.x * 64 + lane, kq = threadIdx.x >> 6;
+    float acc[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = 0.f;
     for (int k0 = 0; k0 < K; k0 += 128) {
         const int kc = min(128, K - k0);
         __syncthreads();
@@ -106,34 +110,40 @@ __global__ __launch_bounds__(256) void head_project_kernel(TO* __restrict__ out,
         }
         __syncthreads();
         if (o < O) {
-            const TW* wp = w + (long)h * w_head + (long)o * w_o + (long)k0 * w_k;
-            for (int k = 0; k < kc; ++k) {
-                const float wv = Io<TW>::ld(wp + (long)k * w_k);
+            const int per = (kc + 3) / 4, ka = kq * per, kb = min(kc, ka + per);
+            const TW* wp = w + ((long)h * K + k0) * O + o;
+            for (int k = ka; k < kb; ++k) {
+                const float wv = Io<TW>::ld(wp + (long)k * O);
 #pragma unroll
-                for (int i = 0; i < 4; ++i) acc[i] += in_s[tg * 4 + i][k] * wv;
+                for (int i = 0; i < 16; ++i) acc[i] += in_s[i][k] * wv;
             }
         }
     }
-    if (o < O) {
+    if (kq > 0) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int t = m0 + tg * 4 + i;
-            if (t < M) Io<TO>::st(out + (long)t * out_ld + (long)h * out_head + o, acc[i]);
+        for (int i = 0; i < 16; ++i) part[kq - 1][i][lane] = acc[i];
+    }
+    __syncthreads();
+    if (kq == 0 && o < O) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int t = m0 + i;
+            if (t < M) Io<TO>::st(out + (long)t * out_ld + (long)h * out_head + o, acc[i] + part[0][i][lane] + part[1][i][lane] + part[2][i][lane]);
         }
     }
 }
 
 // in_wide / out_wide: the activations on that side are 32-bit whatever `dtype` (the type of w) says
 extern "C" int pta_head_project(void* out, int out_wide, long out_ld, long out_head, const void* in, int in_wide,
-                                long in_ld, long in_head, const void* w, long w_head, long w_o, long w_k, int M, int H,
-                                int K, int O, int dtype, void* stream) {
+                                long in_ld, long in_head, const void* w, int M, int H, int K, int O, int dtype,
+                                void* stream) {
     PTA_REQUIRE(M > 0 && H > 0 && K > 0 && O > 0, "head_project: sizes must be positive");
     PTA_REQUIRE(out && in && w, "head_project: null pointer");
     PTA_REQUIRE(H <= 65535 && (M + 15) / 16 <= 65535, "head_project: too many heads or tokens for one launch");
     hipStream_t s = (hipStream_t)stream;
     const dim3 grid((O + 63) / 64, H, (M + 15) / 16), block(256);
 #define HP_LAUNCH(TI, TW, TO) hipLaunchKernelGGL((head_project_kernel<TI, TW, TO>), grid, block, 0, s, (TO*)out, out_ld, out_head, \
-                                                 (const TI*)in, in_ld, in_head, (const TW*)w, w_head, w_o, w_k, M, K, O)
+                                                 (const TI*)in, in_ld, in_head, (const TW*)w, M, K, O)
     if (dtype == PTA_F32) HP_LAUNCH(float, float, float);
     else if (dtype != PTA_BF16) return pta_fail("head_project: unknown dtype %d", dtype);
     else if (in_wide && out_wide) HP_LAUNCH(float, bf16_t, float);

@@ -14,7 +14,7 @@
 
 #include <stdint.h>
 
-#define PTA_ABI_VERSION 10
+#define PTA_ABI_VERSION 11
 
 #ifdef __cplusplus
 extern "C" {
@@ -253,13 +253,15 @@ int pta_scale_f32(float* x, float f, long n, void* stream);
 
 // ---- layers with a state of fixed size per sequence (recurrent.hip) ----------------------------------------------
 int pta_gated_scan(void* y, const void* zxg, long ld, const float* bz, const float* bx, float* state, long state_ld,
-                   const int* cu_tokens, const int* seq_slot, int n_seqs, int W, int dtype, void* stream);
+                   float* chunk_state, float* chunk_decay, const int* cu_tokens, const int* seq_slot, int n_seqs, int W,
+                   int chunk, int max_chunks, int dtype, void* stream);
 int pta_conv_silu(float* out, const void* in, long ld, const float* w, const float* b, float* tail, long tail_ld,
                   const int* cu_tokens, const int* token_seq, const int* seq_slot, int n_seqs, int M, int C, int K,
                   int dtype, void* stream);
 int pta_ssm_scan(float* y, const float* xbc, const void* dt_in, long dt_ld, const float* dt_bias, const float* A_log,
-                 const float* Dp, float* state, long state_ld, const int* cu_tokens, const int* seq_slot, int n_seqs,
-                 int heads, int P, int N, int G, int dtype, void* stream);
+                 const float* Dp, float* state, long state_ld, float* chunk_state, float* chunk_decay,
+                 const int* cu_tokens, const int* seq_slot, int n_seqs, int heads, int P, int N, int G, int chunk,
+                 int max_chunks, int dtype, void* stream);
 
 // ---- attention over a cache of latents (attn_latent.hip) ----------------------------------------------------------
 int pta_attn_latent_sizes_ok(int H, int dn, int dr, int R);
@@ -267,8 +269,7 @@ int pta_latent_prep(float* q_full, void* k_pool, const void* proj, long ld, cons
                     const PtaRotation* rot, const int* token_pos, const int* token_seq, const int* block_table,
                     int bt_stride, int M, int H, int dn, int dr, int R, int write_cache, int dtype, void* stream);
 int pta_head_project(void* out, int out_wide, long out_ld, long out_head, const void* in, int in_wide, long in_ld,
-                     long in_head, const void* w, long w_head, long w_o, long w_k, int M, int H, int K, int O,
-                     int dtype, void* stream);
+                     long in_head, const void* w, int M, int H, int K, int O, int dtype, void* stream);
 int pta_attn_latent(float* out, const float* q, const void* k_pool, const int* block_table, int bt_stride,
                     const int* token_seq, const int* token_pos, int M, int H, int R, int dr, float scale, int dtype,
                     void* stream);

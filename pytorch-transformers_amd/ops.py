@@ -24,7 +24,7 @@ QKV_LAYOUT_CODES = {"grouped": 0, "tail": 1, "interleaved": 2}
 ACT_CODES = {None: 0, "none": 0, "linear": 0, "gelu": 1, "gelu_python": 1, "gelu_new": 2, "gelu_pytorch_tanh": 2,
              "gelu_fast": 2, "gelu_accurate": 2, "quick_gelu": 3, "relu": 4, "relu2": 5, "relu6": 6, "silu": 7, "swish": 7,
              "sigmoid": 8, "tanh": 9, "leaky_relu": 10, "mish": 11, "gelu_10": 12, "laplace": 13}
-ABI_VERSION = 10
+ABI_VERSION = 11
 PAIRING_CODES = {"half": 0, "interleaved": 1}  # PtaPairing: elements (i, i + rotary_dim / 2) or (2i, 2i + 1)
 BIAS_OF_CODES = {"key": 0, "distance": 1}  # PtaBiasOf: the slope times the key's position, or times key - query position
 
@@ -170,8 +170,29 @@ def _entry_cost(name: str, a) -> tuple:
         return gemm(a[6], a[7], a[8], 4)
     if name == "pta_layernorm_sum":
         return ((a[4] + a[7]) * float(a[17]) * a[19] * 4, 0.0)
-    if name in ("pta_attn_mfma", "pta_attn_generic"):
+    if name in ("pta_attn_mfma", "pta_attn_generic", "pta_attn_latent_mfma", "pta_attn_latent"):
         return (float(timing_hint.get("attn_bytes", 0)), float(timing_hint.get("attn_flops", 0)))
+    val = lambda i: float(getattr(a[i], "value", a[i]) or 0)
+    given = lambda i: 1.0 if getattr(a[i], "value", a[i]) else 0.0
+    if name == "pta_rmsnorm":  # what it reads and writes: x (and gate), the residual, the two results
+        M, H, e = val(14), val(15), (4.0 if a[16] == F32 else 2.0)
+        return (M * H * ((4.0 if a[3] else e) + given(5) * e + given(12) * 4.0 + given(1) * 4.0 + given(0) * e), 0.0)
+    if name == "pta_depth_mix":
+        return (val(6) * ((a[5] + 1) * 4.0 + given(1) * 2.0), 0.0)
+    if name == "pta_widen":
+        return (val(2) * 6.0, 0.0)
+    if name == "pta_gated_scan":
+        return (float(timing_hint.get("rows", 0)) * a[12] * 4 * (4.0 if a[15] == F32 else 2.0), 0.0)
+    if name == "pta_conv_silu":
+        return (float(a[11]) * a[12] * ((4.0 if a[14] == F32 else 2.0) + 4.0), 0.0)
+    if name == "pta_ssm_scan":  # the convolution's output in, y out, both 32-bit
+        M, inner = float(timing_hint.get("rows", 0)), float(a[14] * a[15])
+        return (M * (2 * inner + 2 * a[17] * a[16]) * 4.0, 4.0 * M * inner * a[16])
+    if name == "pta_head_project":
+        M, H, K, O = float(a[9]), a[10], a[11], a[12]
+        return (H * K * O * (4.0 if a[13] == F32 else 2.0) + M * H * (K + O) * 4.0, 2.0 * M * H * K * O)
+    if name == "pta_latent_prep":
+        return (float(a[11]) * val(3) * (4.0 if a[17] == F32 else 2.0), 0.0)
     return (0.0, 0.0)
 
 
@@ -1109,7 +1130,11 @@ def _need_state(state: torch.Tensor, row: int, name: str = "state") -> int:
     return int(state.stride(0))
 
 
-def gated_scan(zxg: torch.Tensor, bz, bx, state: torch.Tensor, cu_tokens: torch.Tensor, seq_slot: torch.Tensor) -> torch.Tensor:
+SCAN_CHUNK_TOKENS = 64  # a sequence that brings more than twice as many tokens is cut into chunks that run side by side
+
+
+def gated_scan(zxg: torch.Tensor, bz, bx, state: torch.Tensor, cu_tokens: torch.Tensor, seq_slot: torch.Tensor,
+               max_new: int = 1) -> torch.Tensor:
     """The gated recurrence ``S = (1 - z) S + z c`` over every sequence's tokens of the step, from and into its row
     of ``state`` ``[slots, W]``: ``zxg`` ``[tokens, 3 W]`` holds the gate's and the candidate's pre-activations
     (biases ``bz``, ``bx`` still to add) and the output gate; returns ``S * silu(g)`` ``[tokens, W]``."""
@@ -1125,9 +1150,18 @@ def gated_scan(zxg: torch.Tensor, bz, bx, state: torch.Tensor, cu_tokens: torch.
     _need(cu_tokens, "cu_tokens", torch.int32, (n + 1,))
     state_ld = _need_state(state, W)
     y = torch.empty((M, W), dtype=zxg.dtype, device=zxg.device)
+    timing_hint["rows"] = M
+    chunk, chunks = SCAN_CHUNK_TOKENS, 1
+    if max_new > 2 * chunk:  # (``max_new``: the most tokens any sequence brings)
+        chunks = (int(max_new) + chunk - 1) // chunk
+    chunk_state = chunk_decay = None
+    if chunks > 1:
+        chunk_state = torch.empty((n * chunks, W), dtype=torch.float32, device=zxg.device)
+        chunk_decay = torch.empty((n * chunks, W), dtype=torch.float32, device=zxg.device)
     if M:
         _call("pta_gated_scan", _ptr(y), _ptr(zxg), ctypes.c_long(ld), _ptr(bz), _ptr(bx), _ptr(state),
-              ctypes.c_long(state_ld), _ptr(cu_tokens), _ptr(seq_slot), n, W, dtype_code(zxg.dtype), _stream())
+              ctypes.c_long(state_ld), _ptr(chunk_state), _ptr(chunk_decay), _ptr(cu_tokens), _ptr(seq_slot), n, W, chunk,
+              chunks, dtype_code(zxg.dtype), _stream())
     return y
 
 
@@ -1154,12 +1188,17 @@ def conv_silu(x: torch.Tensor, w: torch.Tensor, b, tail: torch.Tensor, cu_tokens
     return out
 
 
+SSM_CHUNK_TOKENS = 128  # a sequence that brings more than twice as many tokens is cut into chunks that run side by side
+
+
 def ssm_scan(xbc: torch.Tensor, dt: torch.Tensor, dt_bias, a_log, d_skip, state: torch.Tensor, cu_tokens, seq_slot,
-             heads: int, head_dim: int, state_rows: int, groups: int) -> torch.Tensor:
+             heads: int, head_dim: int, state_rows: int, groups: int, max_new: int = 1) -> torch.Tensor:
     """The state-space recurrence per head over every sequence's tokens, from and into its row of ``state``
     ``[slots, heads * state_rows * head_dim]``: ``xbc`` ``[tokens, heads * head_dim + 2 * groups * state_rows]``
     (32-bit: inputs, then B, then C per group), ``dt`` ``[tokens, heads]`` (compute type, may be a block of
-    columns; softplus and ``dt_bias`` are applied here).  Returns y ``[tokens, heads * head_dim]`` in 32-bit."""
+    columns; softplus and ``dt_bias`` are applied here).  ``max_new``: the most tokens any sequence brings; long
+    sequences are walked in chunks side by side (the same sums in another order).  Returns y ``[tokens, heads *
+    head_dim]`` in 32-bit."""
     inner = heads * head_dim
     C = inner + 2 * groups * state_rows
     M = xbc.shape[0]
@@ -1172,10 +1211,18 @@ def ssm_scan(xbc: torch.Tensor, dt: torch.Tensor, dt_bias, a_log, d_skip, state:
     _need(cu_tokens, "cu_tokens", torch.int32, (n + 1,))
     state_ld = _need_state(state, heads * state_rows * head_dim)
     y = torch.empty((M, inner), dtype=torch.float32, device=xbc.device)
+    timing_hint["rows"] = M
+    chunk, chunks = SSM_CHUNK_TOKENS, 1
+    if max_new > 2 * chunk:
+        chunks = (int(max_new) + chunk - 1) // chunk
+    chunk_state = chunk_decay = None
+    if chunks > 1:
+        chunk_state = torch.empty((n * chunks, heads, state_rows, head_dim), dtype=torch.float32, device=xbc.device)
+        chunk_decay = torch.empty((n * chunks, heads), dtype=torch.float32, device=xbc.device)
     if M:
         _call("pta_ssm_scan", _ptr(y), _ptr(xbc), _ptr(dt), ctypes.c_long(dt_ld), _ptr(dt_bias), _ptr(a_log), _ptr(d_skip),
-              _ptr(state), ctypes.c_long(state_ld), _ptr(cu_tokens), _ptr(seq_slot), n, heads, head_dim, state_rows,
-              groups, dtype_code(dt.dtype), _stream())
+              _ptr(state), ctypes.c_long(state_ld), _ptr(chunk_state), _ptr(chunk_decay), _ptr(cu_tokens), _ptr(seq_slot),
+              n, heads, head_dim, state_rows, groups, chunk, chunks, dtype_code(dt.dtype), _stream())
     return y
 
 
@@ -1215,17 +1262,13 @@ def latent_prep(proj: torch.Tensor, w_norm: torch.Tensor, eps: float, inv_freq, 
     return q_full
 
 
-def head_project(x: torch.Tensor, x_head: int, w: torch.Tensor, heads: int, K: int, O: int, transposed: bool,
+def head_project(x: torch.Tensor, x_head: int, w: torch.Tensor, heads: int, K: int, O: int,
                  out: Optional[torch.Tensor] = None, out_head: Optional[int] = None, out_dtype=None) -> torch.Tensor:
-    """A product per head: ``out[t, h, :O] = W_h x[t, h, :K]``.  ``x`` is ``[tokens, >= heads * x_head]`` (rows may
-    lie apart; head h starts at column ``h * x_head``), 32-bit or of w's type.  ``w`` is ``[heads * O, K]``
-    (``transposed=False``: head h's rows are its outputs) or ``[heads * K, O]`` (``transposed=True``: head h's rows
-    are its inputs, the product is with the transpose).  The result goes to ``out`` ``[tokens, >= heads * out_head]``
-    if given (32-bit or w's type), else to a new ``[tokens, heads * O]`` of ``out_dtype`` (default w's type)."""
-    _need(w, "w")
-    if tuple(w.shape) != ((heads * K, O) if transposed else (heads * O, K)):
-        raise KernelError(f"w {tuple(w.shape)} does not hold {heads} heads of {O} x {K}"
-                          + (" (transposed)" if transposed else ""))
+    """A product per head: ``out[t, h, :O] = x[t, h, :K] @ W_h`` with ``w`` ``[heads, K, O]`` (a head's rows are its
+    inputs).  ``x`` is ``[tokens, >= heads * x_head]`` (rows may lie apart; head h starts at column ``h * x_head``),
+    32-bit or of w's type.  The result goes to ``out`` ``[tokens, >= heads * out_head]`` if given (32-bit or w's
+    type), else to a new ``[tokens, heads * O]`` of ``out_dtype`` (default w's type)."""
+    _need(w, "w", None, (heads, K, O))
     M = x.shape[0]
     if x.dim() != 2 or x.stride(1) != 1 or not x.is_cuda or x.shape[1] < (heads - 1) * x_head + K:
         raise KernelError(f"x {tuple(x.shape)} does not hold {heads} heads of {K} elements {x_head} apart")
@@ -1238,13 +1281,24 @@ def head_project(x: torch.Tensor, x_head: int, w: torch.Tensor, heads: int, K: i
         raise KernelError(f"out {tuple(out.shape)} does not hold {heads} heads of {O} elements {out_head} apart")
     if out.dtype not in (torch.float32, w.dtype):
         raise KernelError(f"out must be 32-bit or {w.dtype}, got {out.dtype}")
-    w_head, w_o, w_k = (K * O, 1, O) if transposed else (O * K, K, 1)
     if M:
         _call("pta_head_project", _ptr(out), int(out.dtype == torch.float32), ctypes.c_long(out.stride(0)),
               ctypes.c_long(out_head), _ptr(x), int(x.dtype == torch.float32), ctypes.c_long(x.stride(0)),
-              ctypes.c_long(x_head), _ptr(w), ctypes.c_long(w_head), ctypes.c_long(w_o), ctypes.c_long(w_k), M, heads, K,
-              O, dtype_code(w.dtype), _stream())
+              ctypes.c_long(x_head), _ptr(w), M, heads, K, O, dtype_code(w.dtype), _stream())
     return out
+
+
+HEAD_PROJECT_LIBRARY_ROWS = 64  # bfloat16 steps of more tokens run their per-head products in the vendor library
+
+
+def head_project_library(x3: torch.Tensor, w: torch.Tensor, out_dtype=None) -> torch.Tensor:
+    """The same products for many tokens through the vendor library's batched product: ``x3`` ``[tokens, heads, K]``
+    (any strides) and ``w`` ``[heads, K, O]``, both bfloat16 -> ``[heads, tokens, O]``."""
+    M, H, K = x3.shape
+    with timed("library_mm", float(w.numel()) * 2, 2.0 * M * H * K * w.shape[2]):
+        if out_dtype is None or out_dtype == x3.dtype:
+            return torch.bmm(x3.transpose(0, 1), w)
+        return torch.bmm(x3.transpose(0, 1), w, out_dtype=out_dtype)
 
 
 LATENT_MFMA = os.environ.get("PTA_LATENT_MFMA", "1") != "0"

@@ -57,6 +57,9 @@ class LatentAttentionMixer(Part):
 
     def after_load(self) -> None:
         self.q_down = Linear.stacked(f"{self.name}.q_dkv", [self.q, self.down])  # both read the layer's input
+        # per head, with a head's rows its inputs: the key expansion as the file has it, the value expansion turned
+        self.k_side = self.up_k.view(self.heads, self.dim, self.rank)
+        self.v_side = self.up_v.view(self.heads, self.value_dim, self.rank).transpose(1, 2).contiguous()
 
     def check_sizes(self) -> None:
         problem = ops.latent_sizes_problem(self.heads, self.dim, self.rot_dim, self.rank)
@@ -78,13 +81,21 @@ class LatentAttentionMixer(Part):
                                  1.0 if rot is None else rot.scale, None if rot is None else rot.rotary_dim,
                                  "half" if rot is None else rot.pairing, ctx.token_pos, ctx.token_seq, table, k_pool,
                                  self.heads, self.dim, self.rot_dim, self.rank, write_cache=call.write_cache)
-        M, D = x.shape[0], self.cache_row
+        M, D, H = x.shape[0], self.cache_row, self.heads
+        library = x.dtype == torch.bfloat16 and M > ops.HEAD_PROJECT_LIBRARY_ROWS
         # each head's plain query through the transpose of its key expansion: the first `rank` of its frame
-        ops.head_project(proj, self.dim + self.rot_dim, self.up_k, self.heads, self.dim, self.rank, transposed=True,
-                         out=q_full.view(M, self.heads * D), out_head=D)
+        if library:
+            plain = proj[:, :H * (self.dim + self.rot_dim)].unflatten(1, (H, self.dim + self.rot_dim))[:, :, :self.dim]
+            q_full[:, :, :self.rank].copy_(ops.head_project_library(plain, self.k_side, torch.float32).transpose(0, 1))
+        else:
+            ops.head_project(proj, self.dim + self.rot_dim, self.k_side, H, self.dim, self.rank,
+                             out=q_full.view(M, H * D), out_head=D)
         lat = ops.attn_latent(q_full, k_pool, table, ctx.token_seq, ctx.token_pos, self.rank, self.scale, ctx=ctx)
-        o = ops.head_project(lat.view(M, self.heads * self.rank), self.rank, self.up_v, self.heads, self.rank,
-                             self.value_dim, transposed=False, out_dtype=x.dtype)
+        if library:
+            o = ops.head_project_library(lat.to(x.dtype), self.v_side).transpose(0, 1).reshape(M, H * self.value_dim)
+        else:
+            o = ops.head_project(lat.view(M, H * self.rank), self.rank, self.v_side, H, self.rank, self.value_dim,
+                                 out_dtype=x.dtype)
         return self.out(o, add1=residual)
 
 

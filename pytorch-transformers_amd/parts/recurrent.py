@@ -53,7 +53,7 @@ class GatedScanMixer(Part):
     def forward(self, x: torch.Tensor, ctx: StepContext, call, residual: Optional[torch.Tensor] = None):
         state = ctx.cache.state_layer(call.cache_group, call.cache_layer)
         zxg = self.zxg(x)
-        y = ops.gated_scan(zxg, self.z.bias, self.x.bias, state, ctx.cu_tokens, ctx.seq_slot)
+        y = ops.gated_scan(zxg, self.z.bias, self.x.bias, state, ctx.cu_tokens, ctx.seq_slot, max_new=max(ctx.new_tokens))
         return self.out(y, add1=residual)
 
 
@@ -106,7 +106,8 @@ class StateSpaceMixer(Part):
         xbc = ops.conv_silu(proj[:, self.inner:self.inner + self.channels], self.conv_w, self.conv_b, row[:, cut:],
                             ctx.cu_tokens, ctx.token_seq, ctx.seq_slot)
         y = ops.ssm_scan(xbc, proj[:, self.inner + self.channels:], self.dt_bias, self.a_log, self.d_skip, row[:, :cut],
-                         ctx.cu_tokens, ctx.seq_slot, self.heads, self.head_dim, self.state_rows, self.groups)
+                         ctx.cu_tokens, ctx.seq_slot, self.heads, self.head_dim, self.state_rows, self.groups,
+                         max_new=max(ctx.new_tokens))
         normed = self.norm.apply(y, ctx.dtype, gate=gate)[0]
         return self.out(normed, add1=residual)
 
