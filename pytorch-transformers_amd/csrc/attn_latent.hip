@@ -88,34 +88,43 @@ extern "C" int pta_latent_prep(float* q_full, void* k_pool, const void* proj, lo
 
 // A small product per head: out[t, h, o] = sum_k in[t, h, k] * W[h][k, o], with head h's matrix at w + h * K * O,
 // K-major (its rows are inputs), so that neighbouring threads read neighbouring outputs.
-// A workgroup owns (16 tokens, head, 64 outputs); its four waves take a quarter of K each and add up in LDS in wave
-// order.  K is walked in pieces of 128 that lie in LDS.  For steps of few tokens; prompts in bfloat16 go to the
-// vendor library's batched product instead.
+// A workgroup of eight waves owns (16 tokens, head, 64 outputs); K is walked in pieces of 512 that lie in LDS, a wave
+// takes an eighth of a piece with all its loads of W in flight at once, and the waves add up in LDS in wave order.
+// For steps of few tokens; prompts in bfloat16 go to the vendor library's batched product instead.
+#define HP_WAVES 8
+#define HP_PIECE 512
+#define HP_PER (HP_PIECE / HP_WAVES)
+
 template <typename TI, typename TW, typename TO>
-__global__ __launch_bounds__(256) void head_project_kernel(TO* __restrict__ out, long out_ld, long out_head,
-                                                           const TI* __restrict__ in, long in_ld, long in_head,
-                                                           const TW* __restrict__ w, int M, int K, int O) {
-    __shared__ float in_s[16][128 + 1];
-    __shared__ float part[3][16][64];
+__global__ __launch_bounds__(64 * HP_WAVES) void head_project_kernel(TO* __restrict__ out, long out_ld, long out_head,
+                                                                     const TI* __restrict__ in, long in_ld, long in_head,
+                                                                     const TW* __restrict__ w, int M, int K, int O) {
+    __shared__ float in_s[16][HP_PIECE + 1];
+    __shared__ float part[HP_WAVES - 1][16][64];
     const int h = blockIdx.y, m0 = blockIdx.z * 16, lane = threadIdx.x & 63, o = blockIdx.x * 64 + lane, kq = threadIdx.x >> 6;
     float acc[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[i] = 0.f;
-    for (int k0 = 0; k0 < K; k0 += 128) {
-        const int kc = min(128, K - k0);
+    for (int k0 = 0; k0 < K; k0 += HP_PIECE) {
+        const int kc = min(HP_PIECE, K - k0);
         __syncthreads();
-        for (int i = threadIdx.x; i < 16 * kc; i += 256) {
+        for (int i = threadIdx.x; i < 16 * kc; i += 64 * HP_WAVES) {
             const int t = i / kc, k = i - t * kc;
             in_s[t][k] = m0 + t < M ? Io<TI>::ld(in + (long)(m0 + t) * in_ld + (long)h * in_head + k0 + k) : 0.f;
         }
         __syncthreads();
         if (o < O) {
-            const int per = (kc + 3) / 4, ka = kq * per, kb = min(kc, ka + per);
-            const TW* wp = w + ((long)h * K + k0) * O + o;
-            for (int k = ka; k < kb; ++k) {
-                const float wv = Io<TW>::ld(wp + (long)k * O);
+            const int ka = kq * HP_PER;
+            const TW* wp = w + ((long)h * K + k0 + ka) * O + o;
+            float wv[HP_PER];
 #pragma unroll
-                for (int i = 0; i < 16; ++i) acc[i] += in_s[i][k] * wv;
+            for (int k = 0; k < HP_PER; ++k) wv[k] = ka + k < kc ? Io<TW>::ld(wp + (long)k * O) : 0.f;
+#pragma unroll
+            for (int k = 0; k < HP_PER; ++k) {
+                if (ka + k < kc) {
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) acc[i] += in_s[i][ka + k] * wv[k];
+                }
             }
         }
     }
@@ -128,7 +137,10 @@ __global__ __launch_bounds__(256) void head_project_kernel(TO* __restrict__ out,
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             const int t = m0 + i;
-            if (t < M) Io<TO>::st(out + (long)t * out_ld + (long)h * out_head + o, acc[i] + part[0][i][lane] + part[1][i][lane] + part[2][i][lane]);
+            float v = acc[i];
+#pragma unroll
+            for (int q = 0; q < HP_WAVES - 1; ++q) v += part[q][i][lane];
+            if (t < M) Io<TO>::st(out + (long)t * out_ld + (long)h * out_head + o, v);
         }
     }
 }
@@ -141,7 +153,7 @@ extern "C" int pta_head_project(void* out, int out_wide, long out_ld, long out_h
     PTA_REQUIRE(out && in && w, "head_project: null pointer");
     PTA_REQUIRE(H <= 65535 && (M + 15) / 16 <= 65535, "head_project: too many heads or tokens for one launch");
     hipStream_t s = (hipStream_t)stream;
-    const dim3 grid((O + 63) / 64, H, (M + 15) / 16), block(256);
+    const dim3 grid((O + 63) / 64, H, (M + 15) / 16), block(64 * HP_WAVES);
 #define HP_LAUNCH(TI, TW, TO) hipLaunchKernelGGL((head_project_kernel<TI, TW, TO>), grid, block, 0, s, (TO*)out, out_ld, out_head, \
                                                  (const TI*)in, in_ld, in_head, (const TW*)w, M, K, O)
     if (dtype == PTA_F32) HP_LAUNCH(float, float, float);

@@ -86,10 +86,15 @@ __global__ __launch_bounds__(256) void attn_latent_mfma_kernel(const LatentArgs 
 #pragma unroll
     for (int c = 0; c < DKC; ++c) {
         float v[8];
+        const int el0 = c * 32 + g * 8;
+        if (valid && (D & 3) == 0 && el0 + 8 <= D) {  // sixteen-byte loads where a query's elements line up
+            const float4 lo = *reinterpret_cast<const float4*>(a.q + row_global * D + el0);
+            const float4 hi = *reinterpret_cast<const float4*>(a.q + row_global * D + el0 + 4);
+            v[0] = lo.x * a.scale, v[1] = lo.y * a.scale, v[2] = lo.z * a.scale, v[3] = lo.w * a.scale;
+            v[4] = hi.x * a.scale, v[5] = hi.y * a.scale, v[6] = hi.z * a.scale, v[7] = hi.w * a.scale;
+        } else {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const int el = c * 32 + g * 8 + e;
-            v[e] = (valid && el < D) ? a.q[row_global * D + el] * a.scale : 0.f;
+            for (int e = 0; e < 8; ++e) v[e] = (valid && el0 + e < D) ? a.q[row_global * D + el0 + e] * a.scale : 0.f;
         }
         qf[c].u = make_uint4(lat_pack(v[0], v[1]), lat_pack(v[2], v[3]), lat_pack(v[4], v[5]), lat_pack(v[6], v[7]));
     }

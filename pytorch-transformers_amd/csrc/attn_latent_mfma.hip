@@ -21,22 +21,39 @@ extern "C" int pta_attn_latent_mfma_ok(int R, int D) {
 }
 
 // out[row, :] = sum_s po[row, s, :] e^(pm[row, s] - m) / sum_s pl[row, s] e^(pm[row, s] - m), m = max_s pm[row, s];
-// splits in order.  One workgroup per row (a token's head).
+// splits in order.  One workgroup per row (a token's head); the splits' weights are formed once, in LDS.
+#define LAT_MAX_SPLITS 1024
+
 __global__ void latent_combine_kernel(float* __restrict__ out, const float* __restrict__ po, const float* __restrict__ pm,
                                       const float* __restrict__ pl, int n_splits, int R) {
+    __shared__ float w_s[LAT_MAX_SPLITS];
+    __shared__ float red[16];
     const long row = blockIdx.x;
     const float* m_row = pm + row * n_splits;
     float m = -INFINITY;
-    for (int s = 0; s < n_splits; ++s) m = fmaxf(m, m_row[s]);
+    for (int s = threadIdx.x; s < n_splits; s += blockDim.x) m = fmaxf(m, m_row[s]);
+    m = block_max(m, red);
     float denom = 0.f;
-    for (int s = 0; s < n_splits; ++s) denom += pl[row * n_splits + s] * (m_row[s] == -INFINITY ? 0.f : expf(m_row[s] - m));
+    for (int s = threadIdx.x; s < n_splits; s += blockDim.x) {
+        const float w = m_row[s] == -INFINITY ? 0.f : expf(m_row[s] - m);
+        w_s[s] = w;
+        denom += pl[row * n_splits + s] * w;
+    }
+    denom = block_sum(denom, red);  // (its barriers also publish w_s)
     const float inv = 1.0f / denom;
+    const float* prow = po + row * n_splits * R;
     for (int el = threadIdx.x; el < R; el += blockDim.x) {
         float acc = 0.f;
-        for (int s = 0; s < n_splits; ++s) {
-            const float w = m_row[s] == -INFINITY ? 0.f : expf(m_row[s] - m);
-            if (w != 0.f) acc += po[(row * n_splits + s) * R + el] * w;
+        int s = 0;
+        for (; s + 4 <= n_splits; s += 4) {
+            const float a0 = prow[(long)s * R + el], a1 = prow[(long)(s + 1) * R + el], a2 = prow[(long)(s + 2) * R + el],
+                        a3 = prow[(long)(s + 3) * R + el];
+            acc += a0 * w_s[s];
+            acc += a1 * w_s[s + 1];
+            acc += a2 * w_s[s + 2];
+            acc += a3 * w_s[s + 3];
         }
+        for (; s < n_splits; ++s) acc += prow[(long)s * R + el] * w_s[s];
         out[row * R + el] = acc * inv;
     }
 }
@@ -47,7 +64,7 @@ extern "C" int pta_attn_latent_mfma(float* out, float* po, float* pm, float* pl,
                                     int n_splits, void* stream) {
     PTA_REQUIRE(M > 0 && n_seqs > 0 && max_new > 0 && H > 0 && R > 0 && dr >= 0, "attn_latent_mfma: sizes must be positive");
     PTA_REQUIRE(out && q && k_pool && block_table && cu_tokens && seq_start, "attn_latent_mfma: null pointer");
-    PTA_REQUIRE(n_splits >= 1 && n_splits <= 65535 && n_seqs <= 65535, "attn_latent_mfma: too many key ranges or sequences");
+    PTA_REQUIRE(n_splits >= 1 && n_splits <= LAT_MAX_SPLITS && n_seqs <= 65535, "attn_latent_mfma: too many key ranges or sequences");
     PTA_REQUIRE(n_splits == 1 || (po && pm && pl && split_size > 0 && split_size % LAT_KB == 0),
                 "attn_latent_mfma: key ranges need room for partial results and a size that is a multiple of %d", LAT_KB);
     PTA_REQUIRE(n_splits == 1 || max_new == 1, "attn_latent_mfma: key ranges are for steps of one token per sequence");

@@ -14,7 +14,7 @@
 
 #include <stdint.h>
 
-#define PTA_ABI_VERSION 11
+#define PTA_ABI_VERSION 12
 
 #ifdef __cplusplus
 extern "C" {
@@ -241,10 +241,13 @@ float pta_philox_uniform(uint64_t seed, uint32_t seq, uint32_t step);
 // v = x (* silu(gate)); n = v / sqrt(mean(v^2) + eps) * (offset + w), each of `groups` equal parts of a row by its
 // own mean; out = residual + mult * n where residual is given, else n; written as 32-bit (out_wide) and / or in the
 // compute type (out_narrow).  x is 32-bit if x_wide, else of the compute type; gate is of the compute type;
-// x_ld / gate_ld: distance of their rows; rows (may be null) picks the source rows.
+// x_ld / gate_ld: distance of their rows; rows (may be null) picks the source rows.  With planes (null: none) the
+// result, which out_wide must place as plane count - 1, is followed by the weighted sum of planes 0 .. count - 1
+// (mix_wide in 32-bit; out_narrow then holds the sum, not the result).
 int pta_rmsnorm(void* out_narrow, float* out_wide, const void* x, int x_wide, long x_ld, const void* gate, long gate_ld,
                 const int* rows, const float* w, float offset, int groups, float eps, const float* residual, float mult,
-                int M, int H, int dtype, void* stream);
+                const float* planes, long plane, const float* coef, int count, float* mix_wide, int M, int H, int dtype,
+                void* stream);
 // out[i] = sum_j coef[j] * planes[j * plane + i], j in order; 32-bit and / or compute type
 int pta_depth_mix(float* out_wide, void* out_narrow, const float* planes, long plane, const float* coef, int count,
                   long n, int dtype, void* stream);

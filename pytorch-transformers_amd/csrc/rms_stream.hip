@@ -9,12 +9,16 @@
 #include "pta_kernels.h"
 
 // v = x (* silu(gate)); n = v / sqrt(mean_group(v^2) + eps) * (offset + w); out = residual + mult * n (or n).
+// With `planes` the result (in out_wide) is the last of `count` streams that lie `plane` floats apart, and the launch
+// goes on to their weighted sum (mix_wide, and out_narrow in the compute type), as depth_mix_kernel forms it.
 // One workgroup per (row, group).  TI: type of x (float or the compute type), T: compute type (gate, narrow output).
 template <typename TI, typename T>
 __global__ void rmsnorm_kernel(T* __restrict__ out_narrow, float* __restrict__ out_wide, const TI* __restrict__ x,
                                long x_ld, const T* __restrict__ gate, long gate_ld, const int* __restrict__ rows,
                                const float* __restrict__ w, float offset, int group_len, float eps,
-                               const float* __restrict__ residual, float mult, int H) {
+                               const float* __restrict__ residual, float mult, int H,
+                               const float* __restrict__ planes, long plane, const float* __restrict__ coef, int count,
+                               float* __restrict__ mix_wide) {
     __shared__ float red[16];
     const int m = blockIdx.x, g = blockIdx.y;
     const long src = rows ? rows[m] : m;
@@ -35,31 +39,41 @@ __global__ void rmsnorm_kernel(T* __restrict__ out_narrow, float* __restrict__ o
         float n = v * inv * (offset + w[g * group_len + i]);
         if (residual) n = residual[src * H + (long)g * group_len + i] + mult * n;
         if (out_wide) out_wide[o + i] = n;
+        if (planes) {  // the result is the last of `count` streams: what goes on is their weighted sum, added in order
+            float acc = 0.f;
+#pragma unroll 8
+            for (int j = 0; j + 1 < count; ++j) acc += coef[j] * planes[(long)j * plane + o + i];
+            n = acc + coef[count - 1] * n;
+            mix_wide[o + i] = n;
+        }
         if (out_narrow) Io<T>::st(out_narrow + o + i, n);
     }
 }
 
 extern "C" int pta_rmsnorm(void* out_narrow, float* out_wide, const void* x, int x_wide, long x_ld, const void* gate,
                            long gate_ld, const int* rows, const float* w, float offset, int groups, float eps,
-                           const float* residual, float mult, int M, int H, int dtype, void* stream) {
+                           const float* residual, float mult, const float* planes, long plane, const float* coef,
+                           int count, float* mix_wide, int M, int H, int dtype, void* stream) {
     PTA_REQUIRE(M > 0 && H > 0, "rmsnorm: M=%d H=%d must be positive", M, H);
     PTA_REQUIRE(x && w && (out_narrow || out_wide), "rmsnorm: null pointer");
     PTA_REQUIRE(groups > 0 && H % groups == 0, "rmsnorm: %d features do not split into %d equal groups", H, groups);
     PTA_REQUIRE(groups <= 65535, "rmsnorm: at most 65535 groups, got %d", groups);
     PTA_REQUIRE(x_ld >= H && (!gate || gate_ld >= H), "rmsnorm: rows lie closer together than they are long");
     PTA_REQUIRE(dtype == PTA_F32 || dtype == PTA_BF16, "rmsnorm: unknown dtype %d", dtype);
+    PTA_REQUIRE(!planes || (coef && count >= 1 && mix_wide && out_wide && !rows && plane >= (long)M * H),
+                "rmsnorm: a sum of streams needs their weights, the planes' distance and both 32-bit results");
     hipStream_t s = (hipStream_t)stream;
     const int L = H / groups;
     const dim3 grid(M, groups), block(L >= 2048 ? 512 : L > 64 ? 256 : 64);
     if (dtype == PTA_F32)
         hipLaunchKernelGGL((rmsnorm_kernel<float, float>), grid, block, 0, s, (float*)out_narrow, out_wide,
-                           (const float*)x, x_ld, (const float*)gate, gate_ld, rows, w, offset, L, eps, residual, mult, H);
+                           (const float*)x, x_ld, (const float*)gate, gate_ld, rows, w, offset, L, eps, residual, mult, H, planes, plane, coef, count, mix_wide);
     else if (x_wide)
         hipLaunchKernelGGL((rmsnorm_kernel<float, bf16_t>), grid, block, 0, s, (bf16_t*)out_narrow, out_wide,
-                           (const float*)x, x_ld, (const bf16_t*)gate, gate_ld, rows, w, offset, L, eps, residual, mult, H);
+                           (const float*)x, x_ld, (const bf16_t*)gate, gate_ld, rows, w, offset, L, eps, residual, mult, H, planes, plane, coef, count, mix_wide);
     else
         hipLaunchKernelGGL((rmsnorm_kernel<bf16_t, bf16_t>), grid, block, 0, s, (bf16_t*)out_narrow, out_wide,
-                           (const bf16_t*)x, x_ld, (const bf16_t*)gate, gate_ld, rows, w, offset, L, eps, residual, mult, H);
+                           (const bf16_t*)x, x_ld, (const bf16_t*)gate, gate_ld, rows, w, offset, L, eps, residual, mult, H, planes, plane, coef, count, mix_wide);
     return pta_check_launch("rmsnorm");
 }
 

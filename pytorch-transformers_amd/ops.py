@@ -24,7 +24,7 @@ QKV_LAYOUT_CODES = {"grouped": 0, "tail": 1, "interleaved": 2}
 ACT_CODES = {None: 0, "none": 0, "linear": 0, "gelu": 1, "gelu_python": 1, "gelu_new": 2, "gelu_pytorch_tanh": 2,
              "gelu_fast": 2, "gelu_accurate": 2, "quick_gelu": 3, "relu": 4, "relu2": 5, "relu6": 6, "silu": 7, "swish": 7,
              "sigmoid": 8, "tanh": 9, "leaky_relu": 10, "mish": 11, "gelu_10": 12, "laplace": 13}
-ABI_VERSION = 11
+ABI_VERSION = 12
 PAIRING_CODES = {"half": 0, "interleaved": 1}  # PtaPairing: elements (i, i + rotary_dim / 2) or (2i, 2i + 1)
 BIAS_OF_CODES = {"key": 0, "distance": 1}  # PtaBiasOf: the slope times the key's position, or times key - query position
 
@@ -175,8 +175,9 @@ def _entry_cost(name: str, a) -> tuple:
     val = lambda i: float(getattr(a[i], "value", a[i]) or 0)
     given = lambda i: 1.0 if getattr(a[i], "value", a[i]) else 0.0
     if name == "pta_rmsnorm":  # what it reads and writes: x (and gate), the residual, the two results
-        M, H, e = val(14), val(15), (4.0 if a[16] == F32 else 2.0)
-        return (M * H * ((4.0 if a[3] else e) + given(5) * e + given(12) * 4.0 + given(1) * 4.0 + given(0) * e), 0.0)
+        M, H, e = val(19), val(20), (4.0 if a[21] == F32 else 2.0)
+        return (M * H * ((4.0 if a[3] else e) + given(5) * e + given(12) * 4.0 + given(1) * 4.0 + given(0) * e
+                         + given(14) * 4.0 * a[17]), 0.0)
     if name == "pta_depth_mix":
         return (val(6) * ((a[5] + 1) * 4.0 + given(1) * 2.0), 0.0)
     if name == "pta_widen":
@@ -1044,12 +1045,16 @@ def _rows_of(t: torch.Tensor, name: str, cols: int, dtype=None):
 def rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float, dtype: torch.dtype, *, offset: float = 0.0, groups: int = 1,
             gate: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None,
             residual: Optional[torch.Tensor] = None, mult: float = 1.0, want_wide: bool = False, want_narrow: bool = True,
-            out_wide: Optional[torch.Tensor] = None):
+            out_wide: Optional[torch.Tensor] = None, mix=None):
     """RMS norm in 32-bit: ``n = v / sqrt(mean(v^2) + eps) * (offset + w)`` with ``v = x`` or ``x * silu(gate)``,
     each of ``groups`` equal parts of a row by its own mean square; with ``residual`` (32-bit) the result is
     ``residual + mult * n``.  ``x`` is 32-bit or of the compute type ``dtype`` and its rows may lie apart, as may
     the gate's.  Returns ``(narrow, wide)``: the result in ``dtype`` and in 32-bit (each None unless wanted;
-    ``out_wide``: where to write the 32-bit result).  In a 32-bit model the two are one tensor."""
+    ``out_wide``: where to write the 32-bit result).  In a 32-bit model the two are one tensor.
+
+    ``mix = (planes, coef, count)``: ``out_wide`` is plane ``count - 1`` of ``planes`` ``[>= count, rows, features]``
+    (32-bit), and the launch goes on to ``sum_j coef[j] * planes[j]`` over the first ``count`` planes, in order, as
+    ``depth_mix`` forms it; ``(narrow, wide)`` are then that sum's."""
     H = w.numel()
     _need(w, "weight", torch.float32, (H,))
     x_wide = x.dtype == torch.float32
@@ -1077,10 +1082,23 @@ def rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float, dtype: torch.dtype, *,
     narrow = None
     if want_narrow and not f32:
         narrow = torch.empty((M, H), dtype=dtype, device=x.device)
+    planes = coef = mix_wide = None
+    count = 0
+    if mix is not None:
+        planes, coef, count = mix
+        _need(planes, "planes", torch.float32)
+        _need(coef, "coef", torch.float32, (count,))
+        if (planes.dim() != 3 or tuple(planes.shape[1:]) != (M, H) or not (0 < count <= planes.shape[0]) or rows is not None
+                or out_wide is None or out_wide.data_ptr() != planes[count - 1].data_ptr()):
+            raise KernelError("a sum of streams needs planes [at least count, rows, features] whose plane count - 1 is out_wide")
+        mix_wide = torch.empty((M, H), dtype=torch.float32, device=x.device)
     if M:
         _call("pta_rmsnorm", _ptr(narrow), _ptr(out_wide), _ptr(x), int(x_wide), ctypes.c_long(x_ld), _ptr(gate),
               ctypes.c_long(gate_ld), _ptr(rows), _ptr(w), ctypes.c_float(offset), int(groups), ctypes.c_float(eps),
-              _ptr(residual), ctypes.c_float(mult), M, H, dtype_code(dtype), _stream())
+              _ptr(residual), ctypes.c_float(mult), _ptr(planes), ctypes.c_long(M * H), _ptr(coef), int(count),
+              _ptr(mix_wide), M, H, dtype_code(dtype), _stream())
+    if mix is not None:
+        return (mix_wide if f32 else narrow), mix_wide
     if f32:
         return (out_wide if want_narrow else None), (out_wide if want_wide else None)
     return narrow, (out_wide if want_wide else None)
@@ -1288,7 +1306,7 @@ def head_project(x: torch.Tensor, x_head: int, w: torch.Tensor, heads: int, K: i
     return out
 
 
-HEAD_PROJECT_LIBRARY_ROWS = 64  # bfloat16 steps of more tokens run their per-head products in the vendor library
+HEAD_PROJECT_LIBRARY_ROWS = 0  # bfloat16 steps of more tokens run their per-head products in the vendor library
 
 
 def head_project_library(x3: torch.Tensor, w: torch.Tensor, out_dtype=None) -> torch.Tensor:

@@ -174,16 +174,15 @@ class PostNormBlock(Part):
         last = self.feed_forward is None
         history = x.history
         keep = history.next_plane() if (history is not None and self.depth_mix is not None) else None
+        # the launch that forms the block's result also keeps it as a stream and goes on to the streams' weighted sum
+        mix = self.depth_mix.fused(history) if keep is not None else None
         mixed = self.mixer.forward(x.narrow, ctx, call)
-        narrow, wide = self.norm_mixer.apply(mixed, ctx.dtype, residual=x.wide, mult=self.residual_mult,
-                                             want_wide=True, want_narrow=not last or keep is None,
-                                             out_wide=keep if last else None)
+        narrow, wide = self.norm_mixer.apply(mixed, ctx.dtype, residual=x.wide, mult=self.residual_mult, want_wide=True,
+                                             out_wide=keep if last else None, mix=mix if last else None)
         if not last:
             out = self.feed_forward.forward(narrow, ctx)
             narrow, wide = self.norm_ffn.apply(out, ctx.dtype, residual=wide, mult=self.residual_mult, want_wide=True,
-                                               want_narrow=keep is None, out_wide=keep)
-        if keep is not None:
-            narrow, wide = self.depth_mix.forward(history, ctx.dtype)
+                                               out_wide=keep, mix=mix)
         return WideResidual(wide, narrow, history)
 
 

@@ -50,6 +50,12 @@ class DepthMix(Part):
     def new_history(self, tokens: int, features: int, device) -> StreamHistory:
         return StreamHistory(self.depth, tokens, features, device)
 
+    def fused(self, history: StreamHistory):
+        """What ``ops.rmsnorm(mix=...)`` needs to form this sum in the launch that fills the last stream."""
+        if history.filled != self.index + 2:
+            raise RuntimeError(f"{self.name}: {history.filled} streams are filled, layer {self.index} mixes {self.index + 2}")
+        return (history.planes, self.weight, history.filled)
+
     def forward(self, history: StreamHistory, dtype: torch.dtype):
         """``(narrow, wide)`` of the weighted sum of the streams filled so far, which must be X_0 .. X_(index + 1)."""
         if history.filled != self.index + 2:

@@ -351,8 +351,8 @@ def test_latent_attention_finds_one_far_key(dtype, rel, far):
 # tokens, and six layers stand on each other.  So whole models in bfloat16 are held to a tenth of the largest logit;
 # each mechanism alone is held to the usual 4 %.  A single token whose normalised sublayer output happens to be a
 # small difference of large terms carries several times that, and differently in every schedule (each rounds in
-# other places), so up to a tenth of a request's positions may lie beyond the bound while the request as a whole
-# stays within 8 % in the root mean square.
+# other places), so up to a tenth of a request's positions (or one) may lie beyond the bound while the request as a whole
+# has its median position within the usual 4 %.
 REL_BF16_MODEL = 0.1
 
 
@@ -361,9 +361,10 @@ def assert_model_close(got, want, rel, what):
         return helpers.assert_close(got, want, rel, what)
     assert got.shape == want.shape and torch.isfinite(got).all(), what
     err, scale = (got.double() - want.double()), float(want.abs().max())
-    beyond = (err.abs().max(dim=1)[0] > rel * scale).double().mean()
-    rms = float(err.pow(2).mean().sqrt() / want.double().pow(2).mean().sqrt())
-    assert beyond <= 0.1 and rms <= 0.08, f"{what}: {float(beyond):.2f} of the positions beyond {rel} of the largest logit, rms {rms:.3f}"
+    worst = err.abs().max(dim=1)[0] / scale  # per position
+    beyond, middle = int((worst > rel).sum()), float(worst.median())
+    assert beyond <= max(1, got.shape[0] // 10) and middle <= 0.04, \
+        f"{what}: {beyond} of {got.shape[0]} positions beyond {rel} of the largest logit, the median position at {middle:.3f}"
 
 
 @pytest.mark.parametrize("dtype,rel", [("float32", helpers.REL_F32), ("bfloat16", REL_BF16_MODEL)])
