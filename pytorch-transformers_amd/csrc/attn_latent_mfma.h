@@ -105,28 +105,51 @@ __global__ __launch_bounds__(256) void attn_latent_mfma_kernel(const LatentArgs 
     const int* bt = a.block_table + (long)s * a.bt_stride;
     const bool wide_rows = (D % 8) == 0;
 
-    for (int kb = k_begin; kb < k_end; kb += LAT_KB) {
-        __syncthreads();  // the last block's reads are done
-        // stage 32 cache rows, padded with zeros to DKC * 32 elements (and past the range's end)
-        for (int idx = tid; idx < LAT_KB * DKC * 4; idx += 256) {
-            const int key = idx / (DKC * 4), ch = idx - key * (DKC * 4);
-            const int pos = kb + key;
+    // Staging: a thread owns one of the block's 32 rows (eight threads a row) and every eighth 16-byte piece of it,
+    // so the page is looked up once and all of a block's loads are in flight together; the next block's loads are
+    // issued before this block's arithmetic and land in LDS at the top of the next round.
+    constexpr int PIECES = (DKC * 4 + 7) / 8;  // pieces of a row per thread
+    constexpr bool AHEAD = DKC <= 12;          // (the largest rows leave no registers for a block in flight)
+    const int st_key = tid >> 3, st_ch = tid & 7;
+    uint4 pre[PIECES];
+    auto fetch = [&](int kb) {
+        const int pos = kb + st_key;
+        const bool live = pos < k_end;
+        const bf16_t* src = nullptr;
+        if (live) {
+            const long page = bt[pos / PTA_PAGE];
+            src = a.k_pool + (page * PTA_PAGE + pos % PTA_PAGE) * (long)D;
+        }
+#pragma unroll
+        for (int i = 0; i < PIECES; ++i) {
+            const int ch = st_ch + 8 * i;
             uint4 val = make_uint4(0u, 0u, 0u, 0u);
-            if (pos < k_end && ch * 8 < D) {
-                const long page = bt[pos / PTA_PAGE];
-                const bf16_t* src = a.k_pool + (page * PTA_PAGE + pos % PTA_PAGE) * (long)D + ch * 8;
+            if (live && ch * 8 < D) {
                 if (wide_rows) {
-                    val = *reinterpret_cast<const uint4*>(src);
+                    val = *reinterpret_cast<const uint4*>(src + ch * 8);
                 } else {
                     uint32_t w[4] = {0u, 0u, 0u, 0u};
 #pragma unroll
                     for (int e = 0; e < 8; ++e)
-                        if (ch * 8 + e < D) w[e >> 1] |= (uint32_t)src[e] << ((e & 1) * 16);
+                        if (ch * 8 + e < D) w[e >> 1] |= (uint32_t)src[ch * 8 + e] << ((e & 1) * 16);
                     val = make_uint4(w[0], w[1], w[2], w[3]);
                 }
             }
-            *reinterpret_cast<uint4*>(Ks + key * DP + ch * 8) = val;
+            pre[i] = val;
         }
+    };
+    if (AHEAD && k_begin < k_end) fetch(k_begin);
+
+    for (int kb = k_begin; kb < k_end; kb += LAT_KB) {
+        __syncthreads();  // the last block's reads are done
+        if (!AHEAD) fetch(kb);
+        // 32 cache rows, padded with zeros to DKC * 32 elements (and past the range's end)
+#pragma unroll
+        for (int i = 0; i < PIECES; ++i) {
+            const int ch = st_ch + 8 * i;
+            if (ch < DKC * 4) *reinterpret_cast<uint4*>(Ks + st_key * DP + ch * 8) = pre[i];
+        }
+        if (AHEAD && kb + LAT_KB < k_end) fetch(kb + LAT_KB);
         __syncthreads();
         // the value part transposed: Vt[element][key]; elements past R are never read out of the result
         for (int idx = tid; idx < LAT_KB * RT * 2; idx += 256) {
@@ -138,20 +161,31 @@ __global__ __launch_bounds__(256) void attn_latent_mfma_kernel(const LatentArgs 
                 Vt[(ch * 8 + e) * LAT_VP + key] = (bf16_t)((w[e >> 1] >> ((e & 1) * 16)) & 0xffffu);
         }
         __syncthreads();
-        if (kb > wave_last) continue;  // nothing of this block is visible to this wave's columns
+        if (kb > wave_last || row0 + wave * 16 >= rows_total) continue;  // nothing here for this wave's columns (or it has none)
 
         // scores of 32 keys x 16 columns: tile tt's row i is key 8 * (i / 4) + 4 * tt + i % 4 of the block
+        // (operands come out of LDS in batches ahead of the products that use them: a read that is waited for
+        // in front of every product costs its whole latency each time)
         lat_f32x4_t sc[2];
+        sc[0] = lat_f32x4_t{0.f, 0.f, 0.f, 0.f};
+        sc[1] = lat_f32x4_t{0.f, 0.f, 0.f, 0.f};
+        const bf16_t* krow0 = Ks + (8 * (j >> 2) + (j & 3)) * DP + g * 8;
+        const bf16_t* krow1 = krow0 + 4 * DP;
 #pragma unroll
-        for (int tt = 0; tt < 2; ++tt) {
-            sc[tt] = lat_f32x4_t{0.f, 0.f, 0.f, 0.f};
-            const bf16_t* krow = Ks + (8 * (j >> 2) + 4 * tt + (j & 3)) * DP + g * 8;
+        for (int c0 = 0; c0 < DKC; c0 += 4) {
+            LatFrag kf[2][4];
 #pragma unroll
-            for (int c = 0; c < DKC; ++c) {
-                LatFrag kf;
-                kf.u = *reinterpret_cast<const uint4*>(krow + c * 32);
-                sc[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qf[c].v, sc[tt], 0, 0, 0);
-            }
+            for (int i = 0; i < 4; ++i)
+                if (c0 + i < DKC) {
+                    kf[0][i].u = *reinterpret_cast<const uint4*>(krow0 + (c0 + i) * 32);
+                    kf[1][i].u = *reinterpret_cast<const uint4*>(krow1 + (c0 + i) * 32);
+                }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (c0 + i < DKC) {
+                    sc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[0][i].v, qf[c0 + i].v, sc[0], 0, 0, 0);
+                    sc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[1][i].v, qf[c0 + i].v, sc[1], 0, 0, 0);
+                }
         }
         // the lane holds column j, keys kb + 8 g + 4 tt + r
         float p[8];
@@ -186,14 +220,20 @@ __global__ __launch_bounds__(256) void attn_latent_mfma_kernel(const LatentArgs 
         const bool rescale = __any(corr != 1.f);
         const bf16_t* vrow = Vt + j * LAT_VP + g * 8;
 #pragma unroll
-        for (int dt = 0; dt < RT; ++dt) {
-            if (rescale) {
+        for (int d0 = 0; d0 < RT; d0 += 8) {
+            LatFrag vf[8];
 #pragma unroll
-                for (int r = 0; r < 4; ++r) oacc[dt][r] *= corr;
-            }
-            LatFrag vf;
-            vf.u = *reinterpret_cast<const uint4*>(vrow + dt * 16 * LAT_VP);
-            oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf.v, oacc[dt], 0, 0, 0);
+            for (int i = 0; i < 8; ++i)
+                if (d0 + i < RT) vf[i].u = *reinterpret_cast<const uint4*>(vrow + (d0 + i) * 16 * LAT_VP);
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                if (d0 + i < RT) {
+                    if (rescale) {
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) oacc[d0 + i][r] *= corr;
+                    }
+                    oacc[d0 + i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[i].v, pf.v, oacc[d0 + i], 0, 0, 0);
+                }
         }
     }
     float l_tot = l_run + __shfl_xor(l_run, 16, 64);

@@ -498,3 +498,20 @@ def test_latent_attention_on_matrix_cores_equals_the_32_bit_kernel(heads, rank, 
         want = ops.attn_latent(q, pool, table, seq, pos, rank, 0.2)
         got = ops.attn_latent(q, pool, table, seq, pos, rank, 0.2, ctx=ctx)
         _close(got, want.cpu(), 2e-2, f"latent attention {heads} heads, rows {rank}+{rot}, new tokens {news}")
+
+
+def test_the_command_line_generates_from_a_model_folder(tmp_path, capsys):
+    """``run_generation`` on a folder of this design: greedy tokens as the plain model chooses them."""
+    from pytorch_transformers_amd import run_generation
+
+    cfg = CONFIGS["ones"]
+    w = make_weights(cfg, seed=15)
+    folder = write_model(tmp_path / "m", cfg, w)
+    rc = run_generation.main(["--model_name_or_path", folder, "--model_type", "pavodra", "--prompt_ids", "3,1,4,1,5",
+                              "--length", "6", "--greedy", "--dtype", "float32"])
+    assert rc == 0
+    printed = [ln for ln in capsys.readouterr().out.splitlines() if ln and ln[0].isdigit()]
+    toks = [3, 1, 4, 1, 5]
+    for _ in range(6):
+        toks.append(int(P.forward(cfg, w, toks)[0][-1].argmax()))
+    assert [int(t) for t in printed[-1].split(",")] == toks
