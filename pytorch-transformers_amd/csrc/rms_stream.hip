@@ -50,6 +50,90 @@ __global__ void rmsnorm_kernel(T* __restrict__ out_narrow, float* __restrict__ o
     }
 }
 
+// The same for groups of at most VPT * blockDim elements: a thread keeps its VPT elements in registers between the
+// two passes, and every pass asks for all of its loads before it uses one (a row of a few thousand elements in a
+// step of a few rows is a chain of memory round trips and nothing else).
+template <typename TI, typename T, int VPT>
+__global__ void rmsnorm_reg_kernel(T* __restrict__ out_narrow, float* __restrict__ out_wide, const TI* __restrict__ x,
+                                   long x_ld, const T* __restrict__ gate, long gate_ld, const int* __restrict__ rows,
+                                   const float* __restrict__ w, float offset, int group_len, float eps,
+                                   const float* __restrict__ residual, float mult, int H,
+                                   const float* __restrict__ planes, long plane, const float* __restrict__ coef, int count,
+                                   float* __restrict__ mix_wide) {
+    __shared__ float red[16];
+    const int m = blockIdx.x, g = blockIdx.y;
+    const long src = rows ? rows[m] : m;
+    const TI* xr = x + src * x_ld + (long)g * group_len;
+    const T* gr = gate ? gate + src * gate_ld + (long)g * group_len : nullptr;
+    float v[VPT], z[VPT];
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {
+        const int i = threadIdx.x + k * blockDim.x;
+        v[k] = i < group_len ? Io<TI>::ld(xr + i) : 0.f;
+        z[k] = (gr && i < group_len) ? Io<T>::ld(gr + i) : 0.f;
+    }
+    const long o = (long)m * H + (long)g * group_len;
+    float wv[VPT], rv[VPT];
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {  // asked for now, used after the sum
+        const int i = threadIdx.x + k * blockDim.x;
+        wv[k] = i < group_len ? w[g * group_len + i] : 0.f;
+        rv[k] = (residual && i < group_len) ? residual[src * H + (long)g * group_len + i] : 0.f;
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {
+        if (gr) v[k] *= z[k] / (1.0f + expf(-z[k]));
+        ss += v[k] * v[k];
+    }
+    ss = block_sum(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float)group_len + eps);
+    float n[VPT];
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {
+        n[k] = v[k] * inv * (offset + wv[k]);
+        if (residual) n[k] = rv[k] + mult * n[k];
+    }
+    if (out_wide) {
+#pragma unroll
+        for (int k = 0; k < VPT; ++k) {
+            const int i = threadIdx.x + k * blockDim.x;
+            if (i < group_len) out_wide[o + i] = n[k];
+        }
+    }
+    if (planes) {
+        float acc[VPT];
+#pragma unroll
+        for (int k = 0; k < VPT; ++k) acc[k] = 0.f;
+        for (int j = 0; j + 1 < count; ++j) {
+            const float c = coef[j];
+            const float* pj = planes + (long)j * plane + o;
+            float pv[VPT];
+#pragma unroll
+            for (int k = 0; k < VPT; ++k) {
+                const int i = threadIdx.x + k * blockDim.x;
+                pv[k] = i < group_len ? pj[i] : 0.f;
+            }
+#pragma unroll
+            for (int k = 0; k < VPT; ++k) acc[k] += c * pv[k];
+        }
+        const float c = coef[count - 1];
+#pragma unroll
+        for (int k = 0; k < VPT; ++k) {
+            const int i = threadIdx.x + k * blockDim.x;
+            n[k] = acc[k] + c * n[k];
+            if (i < group_len) mix_wide[o + i] = n[k];
+        }
+    }
+    if (out_narrow) {
+#pragma unroll
+        for (int k = 0; k < VPT; ++k) {
+            const int i = threadIdx.x + k * blockDim.x;
+            if (i < group_len) Io<T>::st(out_narrow + o + i, n[k]);
+        }
+    }
+}
+
 extern "C" int pta_rmsnorm(void* out_narrow, float* out_wide, const void* x, int x_wide, long x_ld, const void* gate,
                            long gate_ld, const int* rows, const float* w, float offset, int groups, float eps,
                            const float* residual, float mult, const float* planes, long plane, const float* coef,
@@ -65,6 +149,15 @@ extern "C" int pta_rmsnorm(void* out_narrow, float* out_wide, const void* x, int
     hipStream_t s = (hipStream_t)stream;
     const int L = H / groups;
     const dim3 grid(M, groups), block(L >= 2048 ? 512 : L > 64 ? 256 : 64);
+#define RMS_ARGS(TN, TX, TG) (TN*)out_narrow, out_wide, (const TX*)x, x_ld, (const TG*)gate, gate_ld, rows, w, offset, L, eps, \
+                             residual, mult, H, planes, plane, coef, count, mix_wide
+    if (L <= 8 * (int)block.x) {  // the group fits the threads' registers
+        if (dtype == PTA_F32) hipLaunchKernelGGL((rmsnorm_reg_kernel<float, float, 8>), grid, block, 0, s, RMS_ARGS(float, float, float));
+        else if (x_wide) hipLaunchKernelGGL((rmsnorm_reg_kernel<float, bf16_t, 8>), grid, block, 0, s, RMS_ARGS(bf16_t, float, bf16_t));
+        else hipLaunchKernelGGL((rmsnorm_reg_kernel<bf16_t, bf16_t, 8>), grid, block, 0, s, RMS_ARGS(bf16_t, bf16_t, bf16_t));
+        return pta_check_launch("rmsnorm");
+    }
+#undef RMS_ARGS
     if (dtype == PTA_F32)
         hipLaunchKernelGGL((rmsnorm_kernel<float, float>), grid, block, 0, s, (float*)out_narrow, out_wide,
                            (const float*)x, x_ld, (const float*)gate, gate_ld, rows, w, offset, L, eps, residual, mult, H, planes, plane, coef, count, mix_wide);
