@@ -107,7 +107,7 @@ __global__ __launch_bounds__(256) void attn_latent_mfma_kernel(const LatentArgs 
 
     // Staging: a thread owns one of the block's 32 rows (eight threads a row) and every eighth 16-byte piece of it,
     // so the page is looked up once and all of a block's loads are in flight together; the next block's loads are
-    // issued before this block's arithmetic and land in LDS at the top of the next round.
+    // issued before this block's arithmetic and land in LDS at the top of the next pass of the loop.
     constexpr int PIECES = (DKC * 4 + 7) / 8;  // pieces of a row per thread
     constexpr bool AHEAD = DKC <= 12;          // (the largest rows leave no registers for a block in flight)
     const int st_key = tid >> 3, st_ch = tid & 7;
