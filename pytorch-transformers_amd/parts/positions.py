@@ -119,7 +119,8 @@ class RotaryPositions(NoPositions):
                 raise ValueError("a rotation of part of a head goes with the default frequencies only")
             if self.rotary_dim < 2 or self.rotary_dim % 2 or self.rotary_dim > head_dim:
                 raise ValueError(f"rotary_dim must be even, from 2 up to the head size {head_dim}; got {rotary_dim}")
-            inv = default_frequencies(self.rotary_dim, self.theta)
+            # (the powers taken in 64-bit and rounded once: a frequency is multiplied by positions in the thousands)
+            inv = (1.0 / (self.theta ** (torch.arange(0, self.rotary_dim, 2, dtype=torch.float64) / self.rotary_dim))).float()
             if self.scaling_factor != 1.0:
                 inv = inv / self.scaling_factor
         elif inv_freq is not None:
