@@ -19,7 +19,7 @@ __global__ void attn_generic_kernel(T* __restrict__ out, const T* __restrict__ q
                                     const T* __restrict__ v_pool, const int* __restrict__ block_table,
                                     int bt_stride, const int* __restrict__ token_seq,
                                     const int* __restrict__ token_pos, const float* __restrict__ slopes, int bias_mode, float bias_scale,
-                                    int nh, int nkv, int d, float scale, int window) {
+                                    int nh, int nkv, int d, float scale, int window, int chunk) {
     __shared__ float q_s[256];
     __shared__ float p_s[PTA_PAGE];
     const int m = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
@@ -33,7 +33,9 @@ __global__ void attn_generic_kernel(T* __restrict__ out, const T* __restrict__ q
     const float slope = slopes ? slopes[h] : 0.f;
 
     // with a window the token sees keys first .. pos only; pages wholly before `first` may be gone
-    const int first = window > 0 ? max(0, nkeys - window) : 0;
+    // with a chunk it sees the keys of its own block of `chunk` positions only
+    int first = window > 0 ? max(0, nkeys - window) : 0;
+    if (chunk > 0) first = max(first, (nkeys - 1) / chunk * chunk);
     float m_run = -INFINITY, l_run = 0.f;
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
     for (int c0 = first / PTA_PAGE * PTA_PAGE; c0 < nkeys; c0 += PTA_PAGE) {
@@ -93,7 +95,7 @@ extern "C" int pta_attention_sizes_ok(int nh, int nkv, int d, int rotated) {
 
 extern "C" int pta_attn_generic(void* out, const void* q, const void* k_pool, const void* v_pool,
                                 const int* block_table, int bt_stride, const int* token_seq, const int* token_pos,
-                                const PtaScoreBias* score_bias, int M, int nh, int nkv, int d, float scale, int window, int dtype,
+                                const PtaScoreBias* score_bias, int M, int nh, int nkv, int d, float scale, int window, int chunk, int dtype,
                                 void* stream) {
     int bias_mode = 0;
     if (pta_score_bias_mode("attn_generic", score_bias, &bias_mode)) return 1;
@@ -104,16 +106,17 @@ extern "C" int pta_attn_generic(void* out, const void* q, const void* k_pool, co
     PTA_REQUIRE(d > 0 && d <= 256, "attn_generic: head size %d is outside 1..256", d);
     PTA_REQUIRE(nh <= 65535, "attn_generic: at most 65535 heads, got %d", nh);
     PTA_REQUIRE(window >= 0, "attn_generic: window must be 0 (none) or positive, got %d", window);
+    PTA_REQUIRE(chunk >= 0, "attn_generic: chunk must be 0 (none) or positive, got %d", chunk);
     hipStream_t s = (hipStream_t)stream;
     dim3 grid(M, nh);
     if (dtype == PTA_F32)
         hipLaunchKernelGGL(attn_generic_kernel<float>, grid, dim3(PTA_WAVE), 0, s, (float*)out, (const float*)q,
                            (const float*)k_pool, (const float*)v_pool, block_table, bt_stride, token_seq, token_pos,
-                           slopes, bias_mode, bias_scale, nh, nkv, d, scale, window);
+                           slopes, bias_mode, bias_scale, nh, nkv, d, scale, window, chunk);
     else if (dtype == PTA_BF16)
         hipLaunchKernelGGL(attn_generic_kernel<bf16_t>, grid, dim3(PTA_WAVE), 0, s, (bf16_t*)out, (const bf16_t*)q,
                            (const bf16_t*)k_pool, (const bf16_t*)v_pool, block_table, bt_stride, token_seq,
-                           token_pos, slopes, bias_mode, bias_scale, nh, nkv, d, scale, window);
+                           token_pos, slopes, bias_mode, bias_scale, nh, nkv, d, scale, window, chunk);
     else
         return pta_fail("attn_generic: unknown dtype %d", dtype);
     return pta_check_launch("attn_generic");

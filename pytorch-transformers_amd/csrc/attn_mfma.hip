@@ -99,7 +99,7 @@ extern "C" int pta_attn_decode_waves_ok(int d, int tiles, int waves) {
 extern "C" int pta_attn_mfma(void* out, const void* q, const void* k_pool, const void* v_pool, const int* block_table,
                              int bt_stride, const int* cu_tokens, const int* seq_start, const PtaScoreBias* score_bias,
                              int n_seqs, int max_new, int M, int nh, int nkv, int d, float scale, int split_size, int n_splits,
-                             float* po, float* pm, float* pl, int window, int decode_tiles, int decode_waves,
+                             float* po, float* pm, float* pl, int window, int chunk, int decode_tiles, int decode_waves,
                              int prompt_wide, void* stream) {
     PTA_REQUIRE(n_seqs > 0 && max_new > 0 && M > 0 && nh > 0 && nkv > 0, "attn_mfma: sizes must be positive");
     int bias_mode = 0;
@@ -110,6 +110,7 @@ extern "C" int pta_attn_mfma(void* out, const void* q, const void* k_pool, const
     PTA_REQUIRE(pta_attn_mfma_supported(d), "attn_mfma: head size %d is not built (16..128 in steps of 16, or 256)", d);
     PTA_REQUIRE(n_splits >= 1 && n_splits <= 1024, "attn_mfma: n_splits must be 1..1024, got %d", n_splits);
     PTA_REQUIRE(window >= 0, "attn_mfma: window must be 0 (none) or positive, got %d", window);
+    PTA_REQUIRE(chunk >= 0, "attn_mfma: chunk must be 0 (none) or positive, got %d", chunk);
     PTA_REQUIRE(n_splits == 1 || (split_size > 0 && split_size % 64 == 0 && po && pm && pl),
                 "attn_mfma: splitting needs a split size that is a multiple of 64 and buffers for partial results");
     PTA_REQUIRE((long)n_seqs * n_splits <= 65535 && nkv <= 65535, "attn_mfma: too many sequences x splits for one launch");
@@ -162,7 +163,7 @@ extern "C" int pta_attn_mfma(void* out, const void* q, const void* k_pool, const
                 "(one wave, or four or eight with up to two tiles)", decode_waves, dct, d);
     const AttnLaunch a{(bf16_t*)out, po, pm, pl, (const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool,
                        block_table, bt_stride, cu_tokens, seq_start, slopes, bias_mode, bias_scale, n_seqs, max_new, nh, nkv, scale,
-                       split_size, n_splits, window, paired, narrow ? decode_waves : 1, s};
+                       split_size, n_splits, window, chunk, paired, narrow ? decode_waves : 1, s};
 #define PTA_ATTN_CASE(DT_)                                                                        \
     case DT_: {                                                                                   \
         const int none = attn_launch_head<DT_>(a, shared, narrow, wide, dct);                     \

@@ -116,9 +116,16 @@ __global__ __launch_bounds__(64 * W * KS, OCC) void attn_mfma_kernel(
     const int* __restrict__ block_table, int bt_stride, const int* __restrict__ cu_tokens,
     const int* __restrict__ seq_start, const float* __restrict__ slopes, int bias_mode, int nh, int nkv, float scale,
     float alibi_mul,
-    int split_size, int n_splits, int window_arg, int paired) {
+    int split_size, int n_splits, int window_arg, int chunk_arg, int paired) {
     constexpr int D = DT * 16;
     const int window = WIN ? window_arg : 0;
+    const int chunk = WIN ? chunk_arg : 0;  // blocks of positions that a token does not see out of (0: none)
+    // the lowest key that a token at position t sees: never decreasing in t
+    auto lowest_key = [&](int t) {
+        int lo = window > 0 ? max(0, t - window + 1) : 0;
+        if (chunk > 0) lo = max(lo, t / chunk * chunk);
+        return lo;
+    };
     constexpr int DS = (DT + 1) / 2;   // 32-wide steps over the head dimension
     constexpr int CHUNKS = D / 8;      // 16-byte chunks in a row of d elements
     static_assert(KS == 1 || W == 1, "waves either share key blocks or divide them");
@@ -154,8 +161,8 @@ __global__ __launch_bounds__(64 * W * KS, OCC) void attn_mfma_kernel(
     const int kv_len = start + n_new;
     // with a window a column at position t sees keys t - window + 1 .. t; this wave starts at the block of
     // the first key its first column sees (earlier pages may be gone), and at its range's start if split
-    const int lo_first = window > 0 ? max(0, start + col0 / g - window + 1) : 0;   // lowest key any column sees
-    const int lo_last = window > 0 ? max(0, max_qpos - window + 1) : 0;            // lowest key the last column sees
+    const int lo_first = WIN ? lowest_key(start + col0 / g) : 0;   // lowest key any column sees
+    const int lo_last = WIN ? lowest_key(max_qpos) : 0;            // lowest key the last column sees
     const int k_begin = max(n_splits > 1 ? split * split_size : 0, lo_first & ~31);
     const int k_end = !active ? 0 : n_splits > 1 ? min(max_qpos + 1, split * split_size + split_size) : max_qpos + 1;
     const int kb_last = (kv_len - 1) & ~31;  // the last block that has a page
@@ -254,7 +261,7 @@ __global__ __launch_bounds__(64 * W * KS, OCC) void attn_mfma_kernel(
             }
             if (MASKED && !interior) {
                 const int lim = min(qpos[ct] + 1, k_end);  // keys below this, and from `lo` on, count for the column
-                const int lo = window > 0 ? qpos[ct] - window + 1 : 0;
+                const int lo = WIN ? lowest_key(max(qpos[ct], 0)) : 0;
 #pragma unroll
                 for (int j = 0; j < 8; ++j)
                     if (kb + 8 * gq + j >= lim || kb + 8 * gq + j < lo) sacc[j >> 2][ct][j & 3] = -INFINITY;
@@ -381,7 +388,7 @@ __global__ __launch_bounds__(64 * W * KS, OCC) void attn_mfma_kernel(
         // (a launch that cuts the keys into ranges walks its own range only)
         const int k_end_wg = n_splits > 1 ? min(start + wg_last_col / g + 1, split * split_size + split_size)
                                           : start + wg_last_col / g + 1;
-        const int k_begin_wg = max(window > 0 ? max(0, start + wg_col0 / g - window + 1) & ~(SK - 1) : 0,
+        const int k_begin_wg = max(WIN ? lowest_key(start + wg_col0 / g) & ~(SK - 1) : 0,
                                    n_splits > 1 ? split * split_size : 0);
         const int ks_last = (kv_len - 1) & ~(SK - 1);  // the last stage that has a page
         static_assert(PER <= 2, "a thread moves at most two pieces of keys and two of values per stage");
@@ -558,6 +565,7 @@ struct AttnLaunch {
     const int *cu_tokens, *seq_start; const float* slopes; int bias_mode; float bias_scale;
     int n_seqs, max_new, nh, nkv; float scale;
     int split_size, n_splits, window;
+    int chunk;   // 0, or the size of the blocks of positions that a token does not see out of
     int paired;  // workgroups take two column groups each, a late one and the early one that mirrors it
     int waves;   // one token per sequence: waves of a workgroup that divide its keys among them
     hipStream_t s;
@@ -574,9 +582,9 @@ static void launch_attn(const AttnLaunch& a) {
     const dim3 grid(paired ? (groups + 1) / 2 : groups, a.nkv, a.n_seqs * a.n_splits);
     // prompts: a kernel with ALiBi and one without; one token per sequence: one kernel that looks
     constexpr int AL0 = W > 1 ? 0 : 2, AL1 = W > 1 ? 1 : 2;
-    auto kern = a.window > 0 ? attn_mfma_kernel<DT, CT, W, true, KS, AL0, OCC> : attn_mfma_kernel<DT, CT, W, false, KS, AL0, OCC>;
+    auto kern = (a.window > 0 || a.chunk > 0) ? attn_mfma_kernel<DT, CT, W, true, KS, AL0, OCC> : attn_mfma_kernel<DT, CT, W, false, KS, AL0, OCC>;
     if (W > 1 && a.slopes)
-        kern = a.window > 0 ? attn_mfma_kernel<DT, CT, W, true, KS, AL1, OCC> : attn_mfma_kernel<DT, CT, W, false, KS, AL1, OCC>;
+        kern = (a.window > 0 || a.chunk > 0) ? attn_mfma_kernel<DT, CT, W, true, KS, AL1, OCC> : attn_mfma_kernel<DT, CT, W, false, KS, AL1, OCC>;
     constexpr size_t lds = key_split_lds(DT, CT, KS);
     if constexpr (lds > 64 * 1024) {  // more than a launch may ask for unless the kernel has been told, once per device
         static bool told[64] = {};
@@ -589,7 +597,7 @@ static void launch_attn(const AttnLaunch& a) {
     }
     hipLaunchKernelGGL(kern, grid, dim3(64 * W * KS), lds, a.s, a.out, a.po, a.pm, a.pl, a.q, a.k_pool, a.v_pool,
                        a.block_table, a.bt_stride, a.cu_tokens, a.seq_start, a.slopes, a.bias_mode, a.nh, a.nkv,
-                       a.scale * PTA_LOG2E, PTA_LOG2E * a.bias_scale, a.split_size, a.n_splits, a.window, paired);
+                       a.scale * PTA_LOG2E, PTA_LOG2E * a.bias_scale, a.split_size, a.n_splits, a.window, a.chunk, paired);
 }
 
 // column tiles (of sixteen query heads of one KV head) that one wave of a decode launch holds at most:

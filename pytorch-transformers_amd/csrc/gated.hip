@@ -1,0 +1,91 @@
+// Element-wise gates between two matrix products.
+//
+// pta_gated_heads:  out[m, h * dv + e] = n(x)[m, h, e] * sigmoid(g[m, h * dv + e]), where x holds heads of dv elements
+//                   in frames x_head apart (an attention result whose frames are wider than its values), and n is
+//                   the identity or an RMS norm over the whole row of heads * dv elements with a weight.
+// pta_glu:          out[m, f] = act(gate[m, f], up[m, f]) for a feed-forward with a gate:
+//                   PTA_GLU_SILU        silu(gate) * up
+//                   PTA_GLU_CLAMPED     g = min(gate, limit), u = clamp(up, -limit, limit): g * sigmoid(alpha g) * (u + 1)
+// Arithmetic in 32-bit, results in the compute type.
+#include "common.h"
+#include "pta_kernels.h"
+
+template <typename T, typename TX>
+__global__ __launch_bounds__(256) void gated_heads_kernel(T* __restrict__ out, const TX* __restrict__ x, long x_ld,
+                                                          int x_head, const T* __restrict__ g, long g_ld,
+                                                          const float* __restrict__ w, float eps, int heads, int dv) {
+    __shared__ float red[16];
+    const int m = blockIdx.x, N = heads * dv;
+    const TX* xr = x + (long)m * x_ld;
+    float inv = 1.f;
+    if (w) {
+        float ss = 0.f;
+        for (int i = threadIdx.x; i < N; i += blockDim.x) {
+            const float v = Io<TX>::ld(xr + (long)(i / dv) * x_head + i % dv);
+            ss += v * v;
+        }
+        inv = rsqrtf(block_sum(ss, red) / (float)N + eps);
+    }
+    for (int i = threadIdx.x; i < N; i += blockDim.x) {
+        float v = Io<TX>::ld(xr + (long)(i / dv) * x_head + i % dv);
+        if (w) v = v * inv * w[i];
+        const float gate = 1.0f / (1.0f + expf(-Io<T>::ld(g + (long)m * g_ld + i)));
+        Io<T>::st(out + (long)m * N + i, v * gate);
+    }
+}
+
+// x: 32-bit (x_f32) or the compute type; g and out in the compute type
+extern "C" int pta_gated_heads(void* out, const void* x, int x_f32, long x_ld, int x_head, const void* g, long g_ld,
+                               const float* w, float eps, int M, int heads, int dv, int dtype, void* stream) {
+    PTA_REQUIRE(M > 0 && heads > 0 && dv > 0, "gated_heads: sizes must be positive");
+    PTA_REQUIRE(out && x && g, "gated_heads: null pointer");
+    PTA_REQUIRE(x_head >= dv && x_ld >= (long)(heads - 1) * x_head + dv && g_ld >= (long)heads * dv,
+                "gated_heads: rows or frames lie closer together than they are long");
+    PTA_REQUIRE(dtype == PTA_F32 || dtype == PTA_BF16, "gated_heads: unknown dtype %d", dtype);
+    hipStream_t s = (hipStream_t)stream;
+    const dim3 grid(M), block(heads * dv >= 1024 ? 256 : 64);
+    if (dtype == PTA_F32)
+        hipLaunchKernelGGL((gated_heads_kernel<float, float>), grid, block, 0, s, (float*)out, (const float*)x, x_ld, x_head,
+                           (const float*)g, g_ld, w, eps, heads, dv);
+    else if (x_f32)
+        hipLaunchKernelGGL((gated_heads_kernel<bf16_t, float>), grid, block, 0, s, (bf16_t*)out, (const float*)x, x_ld, x_head,
+                           (const bf16_t*)g, g_ld, w, eps, heads, dv);
+    else
+        hipLaunchKernelGGL((gated_heads_kernel<bf16_t, bf16_t>), grid, block, 0, s, (bf16_t*)out, (const bf16_t*)x, x_ld,
+                           x_head, (const bf16_t*)g, g_ld, w, eps, heads, dv);
+    return pta_check_launch("gated_heads");
+}
+
+template <typename T>
+__global__ void glu_kernel(T* __restrict__ out, const T* __restrict__ gate, const T* __restrict__ up, long in_ld, int F,
+                           long n, int kind, float alpha, float limit) {
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const long m = i / F, f = i - m * F;
+    float g = Io<T>::ld(gate + m * in_ld + f), u = Io<T>::ld(up + m * in_ld + f);
+    float y;
+    if (kind == PTA_GLU_CLAMPED) {
+        g = fminf(g, limit);
+        u = fminf(fmaxf(u, -limit), limit);
+        y = g / (1.0f + expf(-alpha * g)) * (u + 1.0f);
+    } else {
+        y = g / (1.0f + expf(-g)) * u;
+    }
+    Io<T>::st(out + i, y);
+}
+
+// gate, up: [M, F] with rows in_ld apart (the two halves of one product's rows); out [M, F] dense
+extern "C" int pta_glu(void* out, const void* gate, const void* up, long in_ld, int M, int F, int kind, float alpha,
+                       float limit, int dtype, void* stream) {
+    PTA_REQUIRE(M > 0 && F > 0 && out && gate && up && in_ld >= F, "glu: sizes must be positive and pointers given");
+    PTA_REQUIRE(kind == PTA_GLU_SILU || kind == PTA_GLU_CLAMPED, "glu: kind %d is not built", kind);
+    PTA_REQUIRE(dtype == PTA_F32 || dtype == PTA_BF16, "glu: unknown dtype %d", dtype);
+    hipStream_t s = (hipStream_t)stream;
+    const long n = (long)M * F;
+    const dim3 grid((unsigned)((n + 255) / 256));
+    if (dtype == PTA_F32)
+        hipLaunchKernelGGL(glu_kernel<float>, grid, dim3(256), 0, s, (float*)out, (const float*)gate, (const float*)up, in_ld, F, n, kind, alpha, limit);
+    else
+        hipLaunchKernelGGL(glu_kernel<bf16_t>, grid, dim3(256), 0, s, (bf16_t*)out, (const bf16_t*)gate, (const bf16_t*)up, in_ld, F, n, kind, alpha, limit);
+    return pta_check_launch("glu");
+}

@@ -14,7 +14,7 @@
 
 #include <stdint.h>
 
-#define PTA_ABI_VERSION 12
+#define PTA_ABI_VERSION 13
 
 #ifdef __cplusplus
 extern "C" {
@@ -85,11 +85,13 @@ int pta_attention_sizes_ok(int nh, int nkv, int d, int rotated);
 
 // causal attention of M tokens over their sequences' cache, 32-bit arithmetic
 // window: 0, or the number of last positions a token sees (itself included)
+// chunk: 0, or the size of the blocks of positions, counted from the sequence's start, that a token does not see out
+// of: position i sees j <= i only if floor(i / chunk) == floor(j / chunk)
 // score_bias (null: none): see PtaScoreBias above; with bf16 = 1 the slopes given are expected rounded to bfloat16 too
 int pta_attn_generic(void* out, const void* q, const void* k_pool, const void* v_pool, const int* block_table,
                      int bt_stride, const int* token_seq, const int* token_pos, const PtaScoreBias* score_bias,
                      int M, int nh,
-                     int nkv, int d, float scale, int window, int dtype, void* stream);
+                     int nkv, int d, float scale, int window, int chunk, int dtype, void* stream);
 
 // the same attention for bfloat16 on the matrix cores; cu_tokens [n_seqs + 1] and seq_start [n_seqs] say
 // which tokens are whose and how long each sequence was before the step; max_new bounds a sequence's new
@@ -112,7 +114,8 @@ int pta_attn_decode_shared_ok(int d, int heads_per_kv_head);
 int pta_attn_mfma(void* out, const void* q, const void* k_pool, const void* v_pool, const int* block_table,
                   int bt_stride, const int* cu_tokens, const int* seq_start, const PtaScoreBias* score_bias,
                   int n_seqs, int max_new, int M, int nh, int nkv, int d, float scale, int split_size, int n_splits, float* po,
-                  float* pm, float* pl, int window, int decode_tiles, int decode_waves, int prompt_wide, void* stream);
+                  float* pm, float* pl, int window, int chunk, int decode_tiles, int decode_waves, int prompt_wide,
+                  void* stream);
 
 // C = act(A . W^T + bias) + add1 + add2, all 32-bit, fixed summation order
 int pta_gemm_f32(float* C, const float* A, const float* W, const float* bias, const float* add1, const float* add2,
@@ -276,6 +279,42 @@ int pta_head_project(void* out, int out_wide, long out_ld, long out_head, const 
 int pta_attn_latent(float* out, const float* q, const void* k_pool, const int* block_table, int bt_stride,
                     const int* token_seq, const int* token_pos, int M, int H, int R, int dr, float scale, int dtype,
                     void* stream);
+
+
+// ---- a 32-bit stream with a token-shifted norm at the head of a block (shift_norm.hip) -------------------------------
+int pta_shift_norm(void* a_out, void* m_out, float* x_out, const float* base, const void* t1, const void* t2,
+                   const float* w1, const float* w2, const float* mu, float* state, long state_ld, const int* token_seq,
+                   const int* token_pos, const int* cu_tokens, const int* seq_slot, int n_seqs, int M, int H, float eps,
+                   int several, int dtype, void* stream);
+int pta_wide_sum(float* out, const float* base, const void* t1, const void* t2, long n, int dtype, void* stream);
+
+// ---- normed heads into attention (qk_norm_rope.hip) ------------------------------------------------------------------
+int pta_head_norm_rope_cache(void* q_out, const void* q_in, const void* k_in, const void* v_in, long in_ld,
+                             const float* q_w, const float* k_w, float eps, int v_norm, const PtaRotation* rotation,
+                             const int* token_pos, const int* token_seq, const int* block_table, int bt_stride,
+                             void* k_pool, void* v_pool, int M, int nh, int nkv, int dk, int dv, int D, int write_cache,
+                             int dtype, void* stream);
+
+// ---- gates between two products (gated.hip) ---------------------------------------------------------------------------
+enum PtaGlu { PTA_GLU_SILU = 0, PTA_GLU_CLAMPED = 1 };
+int pta_gated_heads(void* out, const void* x, int x_f32, long x_ld, int x_head, const void* g, long g_ld, const float* w,
+                    float eps, int M, int heads, int dv, int dtype, void* stream);
+int pta_glu(void* out, const void* gate, const void* up, long in_ld, int M, int F, int kind, float alpha, float limit,
+            int dtype, void* stream);
+
+// ---- linear attention with a decay per head (linear_attn.hip) ---------------------------------------------------------
+int pta_decay_scan(float* y, const void* q, const void* k, const void* v, long ld, const float* decay, float* state,
+                   long state_ld, float* chunk_state, const int* cu_tokens, const int* seq_slot, int n_seqs, int heads,
+                   int P, int N, int act, int chunk, int max_chunks, int dtype, void* stream);
+
+// ---- routed experts (moe.hip) -----------------------------------------------------------------------------------------
+enum PtaRouteScore { PTA_ROUTE_SIGMOID = 0, PTA_ROUTE_SOFTMAX = 1 };
+int pta_moe_route(int* ids, float* wts, const void* h, long h_ld, const float* Wr, int M, int H, int E, int top,
+                  int score_kind, int normalise, float scale, int dtype, void* stream);
+int pta_moe_up(void* act_out, const void* h, long h_ld, const void* gate_up, const int* ids, int M, int H, int F, int top,
+               int act, int dtype, void* stream);
+int pta_moe_down(void* out, const void* act_in, const void* down, const int* ids, const float* wts, int M, int H, int F,
+                 int top, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

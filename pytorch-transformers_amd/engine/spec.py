@@ -34,6 +34,9 @@ class TensorSpec:
     #: name is read as before; random weights are drawn and written whole.
     pieces: Tuple[Tuple[str, Tuple[int, ...]], ...] = ()
     assemble: Optional[Callable[[Sequence[Any]], Any]] = None
+    #: the other way round: the pieces, in their order, of a whole tensor.  Given, the writer of random models writes
+    #: the pieces under their names (the layout of the design's files) instead of the whole tensor under its own.
+    split: Optional[Callable[[Any], Sequence[Any]]] = None
 
 
 # kinds of per-sequence storage a group of layers can ask for
@@ -71,6 +74,16 @@ class LayerCall:
     cache_group: Optional[str] = None
     cache_layer: int = 0
     write_cache: bool = True
+    #: further storage of this entry by the name its block knows it under: ``((name, cache group, layer), ...)``,
+    #: for a block that keeps something per sequence beside what its mixer keeps (``also("shift")``)
+    more: Tuple[Tuple[str, str, int], ...] = ()
+
+    def also(self, name: str) -> Tuple[str, int]:
+        """(cache group, layer) of the further storage called ``name``."""
+        for n, group, layer in self.more:
+            if n == name:
+                return group, layer
+        raise KeyError(f"this entry of the run order names no storage {name!r}; it has {[n for n, _, _ in self.more]}")
 
 
 @dataclasses.dataclass
@@ -141,3 +154,8 @@ class ModelSpec:
                 written.add(key)
             elif key not in written:
                 raise ValueError(f"order[{i}] reads cache layer {key} before any entry wrote it")
+            for name, group, layer in call.more:
+                g = groups.get(group)
+                if g is None or not (0 <= layer < g.num_layers):
+                    raise ValueError(f"order[{i}]: storage {name!r} names layer {layer} of cache group {group!r}, which "
+                                     "is not declared")

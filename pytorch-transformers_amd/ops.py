@@ -24,7 +24,7 @@ QKV_LAYOUT_CODES = {"grouped": 0, "tail": 1, "interleaved": 2}
 ACT_CODES = {None: 0, "none": 0, "linear": 0, "gelu": 1, "gelu_python": 1, "gelu_new": 2, "gelu_pytorch_tanh": 2,
              "gelu_fast": 2, "gelu_accurate": 2, "quick_gelu": 3, "relu": 4, "relu2": 5, "relu6": 6, "silu": 7, "swish": 7,
              "sigmoid": 8, "tanh": 9, "leaky_relu": 10, "mish": 11, "gelu_10": 12, "laplace": 13}
-ABI_VERSION = 12
+ABI_VERSION = 13
 PAIRING_CODES = {"half": 0, "interleaved": 1}  # PtaPairing: elements (i, i + rotary_dim / 2) or (2i, 2i + 1)
 BIAS_OF_CODES = {"key": 0, "distance": 1}  # PtaBiasOf: the slope times the key's position, or times key - query position
 
@@ -407,9 +407,11 @@ def attention_sizes_problem(nh: int, nkv: int, d: int, rotated: bool) -> Optiona
 
 
 def attn_generic(q: torch.Tensor, k_pool, v_pool, block_table, token_seq, token_pos, slopes, scale: float,
-                 window: int = 0, alibi_exact: bool = False, bias_of: str = "key", bias_scale: Optional[float] = None):
+                 window: int = 0, alibi_exact: bool = False, bias_of: str = "key", bias_scale: Optional[float] = None,
+                 chunk: int = 0):
     """Causal attention of every token over its sequence's cache (the last ``window`` positions of it, itself
-    included, if ``window`` > 0); out [M, nh*d].  ``slopes`` (None: no bias), ``bias_of``, ``alibi_exact`` (no
+    included, if ``window`` > 0; the positions of its own block of ``chunk``, counted from the sequence's start, if
+    ``chunk`` > 0); out [M, nh*d].  ``slopes`` (None: no bias), ``bias_of``, ``alibi_exact`` (no
     rounding to bfloat16) and ``bias_scale`` (None: 1 / sqrt(head size), as the reference folds its bias into the
     mask) describe a bias on the scores (``_score_bias_arg``)."""
     _need(q, "q")
@@ -423,7 +425,7 @@ def attn_generic(q: torch.Tensor, k_pool, v_pool, block_table, token_seq, token_
     out = torch.empty((M, nh * d), dtype=q.dtype, device=q.device)
     _call("pta_attn_generic", _ptr(out), _ptr(q), _ptr(k_pool), _ptr(v_pool), _ptr(block_table),
           block_table.shape[1], _ptr(token_seq), _ptr(token_pos), bias, M, nh, nkv, d,
-          ctypes.c_float(scale), int(window), dtype_code(q.dtype), _stream())
+          ctypes.c_float(scale), int(window), int(chunk), dtype_code(q.dtype), _stream())
     return out
 
 
@@ -469,7 +471,8 @@ def attn_decode_shared_ok(head_dim: int, heads_per_kv_head: int) -> bool:
 def attn_mfma(q: torch.Tensor, k_pool, v_pool, block_table, cu_tokens, seq_start, slopes, scale: float, *,
               max_new: int, n_splits: int = 1, split_size: int = ATTN_SPLIT_KEYS, window: int = 0,
               decode_tiles: int = 0, decode_waves: int = 1, alibi_exact: bool = False,
-              prompt_wide: Optional[bool] = None, bias_of: str = "key", bias_scale: Optional[float] = None) -> torch.Tensor:
+              prompt_wide: Optional[bool] = None, bias_of: str = "key", bias_scale: Optional[float] = None,
+              chunk: int = 0) -> torch.Tensor:
     """Causal attention of a step's tokens over the cache on the matrix cores; out [M, nh*d].
 
     ``max_new`` bounds the new tokens of any sequence of the step; with ``n_splits > 1`` the keys
@@ -498,15 +501,17 @@ def attn_mfma(q: torch.Tensor, k_pool, v_pool, block_table, cu_tokens, seq_start
     _call("pta_attn_mfma", _ptr(out), _ptr(q), _ptr(k_pool), _ptr(v_pool), _ptr(block_table), block_table.shape[1],
           _ptr(cu_tokens), _ptr(seq_start), bias, n_seqs, int(max_new), M, nh, nkv, d,
           ctypes.c_float(scale),
-          int(split_size), int(n_splits), _ptr(po), _ptr(pm), _ptr(pl), int(window), int(decode_tiles), int(decode_waves),
+          int(split_size), int(n_splits), _ptr(po), _ptr(pm), _ptr(pl), int(window), int(chunk), int(decode_tiles), int(decode_waves),
           ATTN_FORCE_WIDE if prompt_wide is None else int(bool(prompt_wide)), _stream())
     return out
 
 
 
 def attention(q: torch.Tensor, k_pool, v_pool, block_table, ctx, slopes, scale: float, window: int = 0,
-              alibi_exact: bool = False, bias_of: str = "key", bias_scale: Optional[float] = None) -> torch.Tensor:
+              alibi_exact: bool = False, bias_of: str = "key", bias_scale: Optional[float] = None,
+              chunk: int = 0) -> torch.Tensor:
     """Attention of a step's tokens over the cache: picks the kernel for the step's shape and type.
+    ``chunk`` > 0: a token sees the keys of its own block of so many positions only (``attn_generic``).
 
     bfloat16 with a head size the matrix-core kernel is built for: that kernel, with the context
     split over several waves when every sequence brings one token; anything else: the 32-bit
@@ -515,16 +520,16 @@ def attention(q: torch.Tensor, k_pool, v_pool, block_table, ctx, slopes, scale: 
         n_splits, size, tiles, waves = 1, ATTN_SPLIT_KEYS, 0, 1
         if ctx.is_decode:
             shape = (ctx.n_seqs, q.shape[1], k_pool.shape[1], q.shape[2], ctx.max_len, getattr(ctx, "mean_len", 0))
-            if window == 0:
+            if window == 0 and chunk == 0:
                 tuning.note_decode_launch(*shape)
             tiles, size, waves = tuning.decode_plan(*shape)
             n_splits = (ctx.max_len + size - 1) // size
         return attn_mfma(q, k_pool, v_pool, block_table, ctx.cu_tokens, ctx.seq_start, slopes, scale,
                          max_new=max(ctx.new_tokens), n_splits=n_splits, split_size=size, window=window,
                          decode_tiles=tiles, decode_waves=waves, alibi_exact=alibi_exact, bias_of=bias_of,
-                         bias_scale=bias_scale)
+                         bias_scale=bias_scale, chunk=chunk)
     return attn_generic(q, k_pool, v_pool, block_table, ctx.token_seq, ctx.token_pos, slopes, scale, window, alibi_exact,
-                        bias_of, bias_scale)
+                        bias_of, bias_scale, chunk)
 
 
 def sample(logits: torch.Tensor, *, do_sample: bool, temperature: float = 1.0, top_k: int = 0, top_p: float = 1.0,
@@ -1370,4 +1375,193 @@ def attn_latent(q_full: torch.Tensor, k_pool: torch.Tensor, block_table, token_s
     _call("pta_attn_latent", _ptr(out), _ptr(q_full), _ptr(k_pool), _ptr(block_table), block_table.shape[1],
           _ptr(token_seq), _ptr(token_pos), M, H, int(rank), D - int(rank), ctypes.c_float(scale),
           dtype_code(k_pool.dtype), _stream())
+    return out
+
+
+# ---- a 32-bit stream with a token-shifted norm at the head of a block ---------------------------------------------
+def shift_norm(base: torch.Tensor, terms, w1: torch.Tensor, w2: Optional[torch.Tensor], mu: torch.Tensor, eps: float,
+               state: torch.Tensor, ctx, dtype: torch.dtype):
+    """The stream ``x = base + sum(terms)`` (32-bit; ``terms``: up to two tensors of the compute type that a block
+    left), its norm with ``w1`` mixed with the token before's by ``mu`` (``n1 + (n1' - n1) * mu``; the token before
+    a step's first is the sequence's row of ``state``, which is moved on to the step's last), and its norm with
+    ``w2`` (None: none).  Returns ``(x, shifted, second norm or None)``, the last two in ``dtype``."""
+    M, H = base.shape
+    _need(base, "base", torch.float32, (M, H))
+    terms = [t for t in terms if t is not None]
+    if len(terms) > 2:
+        raise KernelError(f"at most two terms are added to the stream, got {len(terms)}")
+    for t in terms:
+        _need(t, "term", dtype, (M, H))
+    for name, t in (("w1", w1), ("mu", mu)) + ((("w2", w2),) if w2 is not None else ()):
+        _need(t, name, torch.float32, (H,))
+    state_ld = _need_state(state, H)
+    n = ctx.seq_slot.numel()
+    _need(ctx.token_seq, "token_seq", torch.int32, (M,))
+    _need(ctx.token_pos, "token_pos", torch.int32, (M,))
+    _need(ctx.cu_tokens, "cu_tokens", torch.int32, (n + 1,))
+    x = torch.empty_like(base) if terms else None
+    a = torch.empty((M, H), dtype=dtype, device=base.device)
+    m = torch.empty((M, H), dtype=dtype, device=base.device) if w2 is not None else None
+    _call("pta_shift_norm", _ptr(a), _ptr(m), _ptr(x), _ptr(base), _ptr(terms[0] if terms else None),
+          _ptr(terms[1] if len(terms) > 1 else None), _ptr(w1), _ptr(w2), _ptr(mu), _ptr(state), ctypes.c_long(state_ld),
+          _ptr(ctx.token_seq), _ptr(ctx.token_pos), _ptr(ctx.cu_tokens), _ptr(ctx.seq_slot), n, M, H, ctypes.c_float(eps),
+          int(max(ctx.new_tokens) > 1), dtype_code(dtype), _stream())
+    return (x if terms else base), a, m
+
+
+def wide_sum(base: torch.Tensor, terms) -> torch.Tensor:
+    """``base + sum(terms)`` in 32-bit (``terms``: one or two tensors of one type, 32-bit or bfloat16)."""
+    terms = [t for t in terms if t is not None]
+    if not terms:
+        return base
+    _need(base, "base", torch.float32)
+    for t in terms:
+        _need(t, "term", terms[0].dtype, tuple(base.shape))
+    out = torch.empty_like(base)
+    _call("pta_wide_sum", _ptr(out), _ptr(base), _ptr(terms[0]), _ptr(terms[1] if len(terms) > 1 else None),
+          ctypes.c_long(base.numel()), dtype_code(terms[0].dtype), _stream())
+    return out
+
+
+# ---- normed heads into attention ------------------------------------------------------------------------------------
+def head_norm_rope_cache(q_in: torch.Tensor, k_in: torch.Tensor, v_in: torch.Tensor, q_w, k_w, eps: float, v_norm: bool,
+                         rotation, ctx, block_table, k_pool, v_pool, nh: int, nkv: int, dk: int, dv: int,
+                         write_cache: bool = True) -> torch.Tensor:
+    """Queries ``[M, nh, D]`` from ``q_in`` ``[M, nh * dk]``; keys (``k_in`` ``[M, nkv * dk]``) and values (``v_in``
+    ``[M, nkv * dv]``) go to the cache pages, whose heads have D >= max(dk, dv) elements (what lies past a head's own
+    is written as zeros).  The three inputs are blocks of columns of one product.  Every query and key head is
+    divided by its root mean square (+ ``eps`` inside the root) and multiplied by ``q_w`` / ``k_w`` ``[dk]`` (None:
+    left as it is), then rotated (``rotation``: a ``parts.positions.Rotation`` or None); every value head is
+    divided by its root mean square if ``v_norm``."""
+    M = q_in.shape[0]
+    dt = q_in.dtype
+    ld = _rows_of(q_in, "q_in", nh * dk, dt)
+    if _rows_of(k_in, "k_in", nkv * dk, dt) != ld or _rows_of(v_in, "v_in", nkv * dv, dt) != ld:
+        if M > 1:
+            raise KernelError("queries, keys and values must be blocks of columns of one matrix")
+    D = k_pool.shape[-1]
+    _need_pools(k_pool, v_pool, dt, nkv, D)
+    for name, t in (("q_w", q_w), ("k_w", k_w)):
+        if t is not None:
+            _need(t, name, torch.float32, (dk,))
+    _need(block_table, "block_table", torch.int32)
+    rot = None
+    if rotation is not None:
+        rot = _rotation_arg(rotation.inv_freq, rotation.scale, dk, block_table.shape[0], rotation.rotary_dim, rotation.pairing)
+    q = torch.empty((M, nh, D), dtype=dt, device=q_in.device)
+    _call("pta_head_norm_rope_cache", _ptr(q), _ptr(q_in), _ptr(k_in), _ptr(v_in), ctypes.c_long(ld), _ptr(q_w), _ptr(k_w),
+          ctypes.c_float(eps), int(bool(v_norm)), rot, _ptr(ctx.token_pos), _ptr(ctx.token_seq), _ptr(block_table),
+          block_table.shape[1], _ptr(k_pool), _ptr(v_pool), M, nh, nkv, dk, dv, D, int(write_cache), dtype_code(dt), _stream())
+    return q
+
+
+# ---- gates between two products -------------------------------------------------------------------------------------
+GLU_CODES = {"silu": 0, "clamped": 1}
+
+
+def gated_heads(x: torch.Tensor, x_head: int, g: torch.Tensor, heads: int, dv: int, dtype: torch.dtype,
+                w: Optional[torch.Tensor] = None, eps: float = 0.0) -> torch.Tensor:
+    """``n(x) * sigmoid(g)`` ``[M, heads * dv]`` in ``dtype``: ``x`` (32-bit or ``dtype``) holds heads of ``dv``
+    elements in frames ``x_head`` apart; n is an RMS norm over the row of all heads with the weight ``w``, or the
+    identity (``w`` None); ``g`` ``[M, heads * dv]`` (``dtype``) may be a block of columns."""
+    M = x.shape[0]
+    if x.dim() != 2 or x.stride(1) != 1 or x.shape[1] < (heads - 1) * x_head + dv or x.dtype not in (torch.float32, dtype):
+        raise KernelError(f"x must be [M, at least {(heads - 1) * x_head + dv}] in 32-bit or {dtype}")
+    g_ld = _rows_of(g, "g", heads * dv, dtype)
+    if w is not None:
+        _need(w, "w", torch.float32, (heads * dv,))
+    out = torch.empty((M, heads * dv), dtype=dtype, device=x.device)
+    if M:
+        _call("pta_gated_heads", _ptr(out), _ptr(x), int(x.dtype == torch.float32), ctypes.c_long(x.stride(0)), int(x_head),
+              _ptr(g), ctypes.c_long(g_ld), _ptr(w), ctypes.c_float(eps), M, heads, dv, dtype_code(dtype), _stream())
+    return out
+
+
+def glu(gate: torch.Tensor, up: torch.Tensor, kind: str = "silu", alpha: float = 1.0, limit: float = 0.0) -> torch.Tensor:
+    """``silu(gate) * up`` (``"silu"``), or with ``g = min(gate, limit)``, ``u = clamp(up, -limit, limit)``:
+    ``g * sigmoid(alpha * g) * (u + 1)`` (``"clamped"``); gate and up are blocks of columns of one product."""
+    M, F = gate.shape
+    ld = _rows_of(gate, "gate", F)
+    if _rows_of(up, "up", F, gate.dtype) != ld and M > 1:
+        raise KernelError("gate and up must be blocks of columns of one matrix")
+    out = torch.empty((M, F), dtype=gate.dtype, device=gate.device)
+    if M:
+        _call("pta_glu", _ptr(out), _ptr(gate), _ptr(up), ctypes.c_long(ld), M, F, GLU_CODES[kind], ctypes.c_float(alpha),
+              ctypes.c_float(limit), dtype_code(gate.dtype), _stream())
+    return out
+
+
+# ---- linear attention with a decay per head -------------------------------------------------------------------------
+DECAY_SCAN_CHUNK_TOKENS = 128  # a sequence that brings more than twice as many tokens is cut into chunks that run side by side
+
+
+def decay_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Tensor, state: torch.Tensor, cu_tokens,
+               seq_slot, heads: int, key_dim: int, value_dim: int, act: Optional[str] = "silu", max_new: int = 1) -> torch.Tensor:
+    """Per head ``S <- decay[h] S + k v^T``, ``o = S^T q`` over every sequence's tokens, from and into its row of
+    ``state`` ``[slots, heads * key_dim * value_dim]`` (32-bit); ``q``, ``k`` ``[tokens, heads * key_dim]`` and ``v``
+    ``[tokens, heads * value_dim]`` are blocks of columns of one product in the compute type, and ``act`` is applied
+    to them on the way in.  Returns o ``[tokens, heads * value_dim]`` in 32-bit."""
+    M = q.shape[0]
+    ld = _rows_of(q, "q", heads * key_dim)
+    if (_rows_of(k, "k", heads * key_dim, q.dtype) != ld or _rows_of(v, "v", heads * value_dim, q.dtype) != ld) and M > 1:
+        raise KernelError("q, k and v must be blocks of columns of one matrix")
+    _need(decay, "decay", torch.float32, (heads,))
+    n = seq_slot.numel()
+    _need(seq_slot, "seq_slot", torch.int32, (n,))
+    _need(cu_tokens, "cu_tokens", torch.int32, (n + 1,))
+    state_ld = _need_state(state, heads * key_dim * value_dim)
+    y = torch.empty((M, heads * value_dim), dtype=torch.float32, device=q.device)
+    chunk, chunks = DECAY_SCAN_CHUNK_TOKENS, 1
+    if max_new > 2 * chunk:
+        chunks = (int(max_new) + chunk - 1) // chunk
+    chunk_state = None
+    if chunks > 1:
+        chunk_state = torch.empty((n * chunks, heads, key_dim, value_dim), dtype=torch.float32, device=q.device)
+    if M:
+        _call("pta_decay_scan", _ptr(y), _ptr(q), _ptr(k), _ptr(v), ctypes.c_long(ld), _ptr(decay), _ptr(state),
+              ctypes.c_long(state_ld), _ptr(chunk_state), _ptr(cu_tokens), _ptr(seq_slot), n, heads, value_dim, key_dim,
+              ACT_CODES[act], chunk, chunks, dtype_code(q.dtype), _stream())
+    return y
+
+
+# ---- routed experts ---------------------------------------------------------------------------------------------------
+ROUTE_SCORE_CODES = {"sigmoid": 0, "softmax": 1}
+
+
+def moe_route(h: torch.Tensor, router: torch.Tensor, top: int, score: str = "sigmoid", normalise: bool = True,
+              scale: float = 1.0):
+    """Per token the ``top`` experts with the largest scores of ``router @ h`` (32-bit; ``router`` ``[experts,
+    features]`` 32-bit) and their weights: ``(ids [M, top] int32, weights [M, top] 32-bit)``."""
+    M, H = h.shape
+    E = router.shape[0]
+    _need(router, "router", torch.float32, (E, H))
+    ld = _rows_of(h, "h", H)
+    ids = torch.empty((M, top), dtype=torch.int32, device=h.device)
+    wts = torch.empty((M, top), dtype=torch.float32, device=h.device)
+    if M:
+        _call("pta_moe_route", _ptr(ids), _ptr(wts), _ptr(h), ctypes.c_long(ld), _ptr(router), M, H, E, int(top),
+              ROUTE_SCORE_CODES[score], int(bool(normalise)), ctypes.c_float(scale), dtype_code(h.dtype), _stream())
+    return ids, wts
+
+
+def moe_experts(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor,
+                act: str = "silu") -> torch.Tensor:
+    """``sum_k wts[m, k] * down[e] (act(gate[e] h) * (up[e] h))`` with ``e = ids[m, k]``: ``gate_up`` ``[experts, 2 F,
+    features]`` (an expert's gate rows, then its up rows), ``down`` ``[experts, features, F]``; out ``[M, features]``."""
+    M, H = h.shape
+    E, F2, _ = gate_up.shape
+    F = F2 // 2
+    top = ids.shape[1]
+    _need(gate_up, "gate_up", h.dtype, (E, 2 * F, H))
+    _need(down, "down", h.dtype, (E, H, F))
+    _need(ids, "ids", torch.int32, (M, top))
+    _need(wts, "wts", torch.float32, (M, top))
+    ld = _rows_of(h, "h", H, h.dtype)
+    act_buf = torch.empty((M * top, F), dtype=h.dtype, device=h.device)
+    out = torch.empty((M, H), dtype=h.dtype, device=h.device)
+    if M:
+        _call("pta_moe_up", _ptr(act_buf), _ptr(h), ctypes.c_long(ld), _ptr(gate_up), _ptr(ids), M, H, F, top,
+              ACT_CODES[act], dtype_code(h.dtype), _stream())
+        _call("pta_moe_down", _ptr(out), _ptr(act_buf), _ptr(down), _ptr(ids), _ptr(wts), M, H, F, top,
+              dtype_code(h.dtype), _stream())
     return out

@@ -4,8 +4,10 @@ from .linear import Embedding, Linear, OutputHead, QkvTail, TailDone
 from .norms import LayerNorm, RMSNorm
 from .positions import AlibiPositions, NoPositions, Rotation, RotaryPositions, ScoreBias, alibi_slopes
 from .attention import AttentionMixer
-from .feedforward import DenseFeedForward
-from .blocks import ParallelBlock, PostNormBlock, SequentialBlock
+from .feedforward import DenseFeedForward, GatedFeedForward, RoutedFeedForward
+from .blocks import ParallelBlock, PostNormBlock, SequentialBlock, ShiftedParallelBlock
+from .gated_attention import GatedAttentionMixer
+from .linear_attention import DecayLinearAttentionMixer
 from .depth import DepthMix
 from .latent_attention import LatentAttentionMixer
 from .recurrent import GatedScanMixer, StateSpaceMixer
@@ -13,4 +15,5 @@ from .recurrent import GatedScanMixer, StateSpaceMixer
 __all__ = ["Part", "StepContext", "make_part", "register_part", "registered_parts", "Embedding", "Linear",
            "OutputHead", "LayerNorm", "AlibiPositions", "NoPositions", "Rotation", "RotaryPositions", "ScoreBias", "alibi_slopes",
            "AttentionMixer", "DenseFeedForward", "ParallelBlock", "SequentialBlock", "PostNormBlock", "RMSNorm", "DepthMix",
-           "LatentAttentionMixer", "GatedScanMixer", "StateSpaceMixer"]
+           "LatentAttentionMixer", "GatedScanMixer", "StateSpaceMixer", "GatedFeedForward", "RoutedFeedForward",
+           "ShiftedParallelBlock", "GatedAttentionMixer", "DecayLinearAttentionMixer"]

@@ -149,6 +149,29 @@ class WideResidual:
         self.wide, self.narrow, self.history = wide, narrow, history
 
 
+class WideSum(WideResidual):
+    """A 32-bit stream as a sum that is not formed yet: ``base`` (32-bit) plus the ``terms`` (up to two tensors of
+    the compute type) that a block's branches left.  The block that runs next forms the sum in the launch that norms
+    it (``ops.shift_norm``); anyone else who asks for ``wide`` (the final norm, a hook) has it formed then."""
+
+    def __init__(self, base: torch.Tensor, terms: Sequence[torch.Tensor], dtype: torch.dtype):
+        self.base, self.terms, self.dtype = base, [t for t in terms if t is not None], dtype
+        self.history = None
+        self._wide = None
+
+    @property
+    def wide(self) -> torch.Tensor:
+        if self._wide is None:
+            from .. import ops
+
+            self._wide = ops.wide_sum(self.base, self.terms)
+        return self._wide
+
+    @property
+    def narrow(self) -> torch.Tensor:
+        return self.wide if self.dtype == torch.float32 else self.wide.to(self.dtype)
+
+
 def as_tensor(x):
     """A tensor from what a part may hand on: a tensor, a ``PartialProduct``, a ``ResidualSum`` or a
     ``WideResidual`` (its 32-bit side)."""

@@ -17,7 +17,8 @@ from typing import Optional, Sequence
 
 import torch
 
-from .base import Part, ResidualSum, StepContext, WideResidual, as_tensor, register_part
+from ..engine.spec import INIT_ZERO_NOISE, VECTOR, TensorSpec
+from .base import Part, ResidualSum, StepContext, WideResidual, WideSum, as_tensor, register_part
 from .linear import Linear, PendingProjection
 
 
@@ -186,6 +187,64 @@ class PostNormBlock(Part):
         return WideResidual(wide, narrow, history)
 
 
+class ShiftedParallelBlock(Part):
+    """``x <- x + (mixer(shift(norm_mixer(x))) + ffn(norm_ffn(x)))`` over a stream kept in 32-bit: both branches read
+    norms of the same x.  ``shift``: what the mixer reads, ``h = norm_mixer(x)``, is replaced by ``h + (h' - h) * mu``
+    with h' the h of the token before (zeros at a sequence's first token) and ``mu`` a learned vector (``shift_name``
+    in the file).  The h of a sequence's last token is part of its state: a row of the state table that the run
+    order's entry names as ``also("shift")``.  ``feed_forward`` may be None (a layer of the mixer alone).
+
+    The block hands on ``x`` and its branches' results as a sum that is not formed (``WideSum``); the next block's
+    first launch forms it, norms it twice and shifts (``ops.shift_norm``)."""
+
+    accepts_sum = False
+    accepts_wide = True
+
+    def __init__(self, mixer: Part, feed_forward: Optional[Part], norm_mixer: Part, norm_ffn: Optional[Part],
+                 shift_name: str, hidden_size: int):
+        if (feed_forward is None) != (norm_ffn is None):
+            raise ValueError("a feed-forward and its norm come together or not at all")
+        if getattr(norm_mixer, "offset", 0.0) or getattr(norm_mixer, "groups", 1) != 1 or (
+                norm_ffn is not None and (norm_ffn.offset or norm_ffn.groups != 1 or norm_ffn.eps != norm_mixer.eps)):
+            raise ValueError("the shifted block's launch takes plain RMS norms with one eps")
+        self.mixer, self.feed_forward, self.norm_mixer, self.norm_ffn = mixer, feed_forward, norm_mixer, norm_ffn
+        self.shift_name, self.hidden_size = shift_name, int(hidden_size)
+        self.mu: Optional[torch.Tensor] = None
+
+    def children(self) -> Sequence[Part]:
+        return tuple(p for p in (self.norm_mixer, self.norm_ffn, self.mixer, self.feed_forward) if p is not None)
+
+    def tensor_specs(self):
+        return [TensorSpec(self.shift_name, (self.hidden_size,), VECTOR, INIT_ZERO_NOISE)]
+
+    def load(self, tensors) -> None:
+        self.mu = tensors[self.shift_name]
+
+    def after_load(self) -> None:
+        for part in (self.mixer, self.feed_forward):
+            if part is not None and hasattr(part, "after_load"):
+                part.after_load()
+
+    def forward(self, x, ctx: StepContext, call):
+        from .. import ops
+
+        if isinstance(x, WideSum):
+            base, terms = x.base, x.terms
+        elif isinstance(x, WideResidual):
+            base, terms = x.wide, []
+        else:
+            x = as_tensor(x)
+            base, terms = (x if x.dtype == torch.float32 else ops.widen(x)), []
+        group, layer = call.also("shift")
+        state = ctx.cache.state_layer(group, layer)
+        stream, a, m = ops.shift_norm(base, terms, self.norm_mixer.weight, None if self.norm_ffn is None else self.norm_ffn.weight,
+                                      self.mu, self.norm_mixer.eps, state, ctx, ctx.dtype)
+        mixed = self.mixer.forward(a, ctx, call)
+        ff = self.feed_forward.forward(m, ctx) if self.feed_forward is not None else None
+        return WideSum(stream, [mixed, ff], ctx.dtype)
+
+
+register_part("block", "shifted_parallel", ShiftedParallelBlock)
 register_part("block", "post_norm", PostNormBlock)
 register_part("block", "parallel", ParallelBlock)
 register_part("block", "sequential", SequentialBlock)

@@ -4,11 +4,12 @@ reference's by name (src/transformers/activations.py:200-220; ``gelu`` is the ex
 in 32-bit in the epilogue of the first product."""
 from __future__ import annotations
 
-from typing import Sequence
+from typing import Dict, List, Optional, Sequence
 
 import torch
 
 from .. import ops
+from ..engine.spec import INIT_NORMAL, MATRIX, VECTOR, TensorSpec
 from .base import Part, StepContext, as_tensor, register_part
 from .linear import Linear, PendingProjection
 
@@ -44,4 +45,104 @@ class DenseFeedForward(Part):
         return self.down(h, add1=as_tensor(add1), add2=as_tensor(add2))
 
 
+class GatedFeedForward(Part):
+    """A feed-forward with a gate: ``down(glu(gate(x), up(x)))``, no biases.  ``kind`` ``"silu"``: ``silu(gate) * up``;
+    ``"clamped"``: with ``g = min(gate, limit)`` and ``u = clamp(up, -limit, limit)``, ``g * sigmoid(alpha * g) * (u +
+    1)``.  The two input products run as one; the gate's arithmetic is 32-bit.  The file holds the matrices as
+    ``name.gate``, ``name.up`` and ``name.down``."""
+
+    def __init__(self, name: str, hidden_size: int, ffn_size: int, kind: str = "silu", alpha: float = 1.0,
+                 limit: float = 0.0):
+        if kind not in ops.GLU_CODES:
+            raise ValueError(f"{name}: a gate of kind {kind!r} is not built; built: {sorted(ops.GLU_CODES)}")
+        self.name, self.kind, self.alpha, self.limit = name, kind, float(alpha), float(limit)
+        self.ffn_size = int(ffn_size)
+        bare = lambda short, i, o: Linear(f"{name}.{short}", i, o, False, weight_name=f"{name}.{short}")
+        self.gate = bare("gate", hidden_size, ffn_size)
+        self.up = bare("up", hidden_size, ffn_size)
+        self.down = bare("down", ffn_size, hidden_size)
+        self.inp: Optional[Linear] = None
+
+    def children(self) -> Sequence[Part]:
+        return (self.gate, self.up, self.down)
+
+    def after_load(self) -> None:
+        self.inp = Linear.stacked(f"{self.name}.gate_up", [self.gate, self.up])
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, add1=None, add2=None):
+        both = self.inp(x)
+        F = self.ffn_size
+        y = ops.glu(both[:, :F], both[:, F:], self.kind, self.alpha, self.limit)
+        return self.down(y, add1=as_tensor(add1), add2=as_tensor(add2))
+
+
+def _stack_experts(experts: int, rows_each: Sequence[int]):
+    """Pieces given expert by expert (each expert's matrices in turn) -> one tensor ``[experts, sum(rows), columns]``."""
+    per = len(rows_each)
+
+    def assemble(parts):
+        return torch.stack([torch.cat(list(parts[e * per:(e + 1) * per]), dim=0) for e in range(experts)])
+
+    return assemble
+
+
+def _unstack_experts(rows_each: Sequence[int]):
+    """The inverse of ``_stack_experts``: ``[experts, sum(rows), columns]`` -> the pieces, expert by expert."""
+
+    def split(t):
+        return [piece for e in range(t.shape[0]) for piece in torch.split(t[e], list(rows_each), dim=0)]
+
+    return split
+
+
+class RoutedFeedForward(Part):
+    """A feed-forward of ``experts`` small gated feed-forwards of which each token uses ``top``:
+
+        z = W_router x (32-bit), s = sigmoid(z) (or softmax(z)); the ``top`` largest s are taken;
+        weight_e = s_e / (sum of the taken s + 1e-20) * scale     (``normalise=False``: s_e * scale)
+        out = sum over the taken e of weight_e * down_e(act(gate_e x) * up_e(x))
+
+    The file holds ``name.router`` ``[experts, hidden]`` and per expert ``name.e<j>.gate``, ``.up`` ``[ff, hidden]``
+    and ``.down`` ``[hidden, ff]``; on the device the experts' matrices are stacked (gate rows then up rows per
+    expert, and the down matrices) and the router is 32-bit."""
+
+    def __init__(self, name: str, hidden_size: int, ffn_size: int, experts: int, top: int, scale: float = 1.0,
+                 score: str = "sigmoid", normalise: bool = True, act: str = "silu"):
+        if not (0 < top <= experts):
+            raise ValueError(f"{name}: {top} of {experts} experts per token")
+        if score not in ops.ROUTE_SCORE_CODES:
+            raise ValueError(f"{name}: router scores of kind {score!r} are not built; built: {sorted(ops.ROUTE_SCORE_CODES)}")
+        self.name, self.hidden_size, self.ffn_size = name, int(hidden_size), int(ffn_size)
+        self.experts, self.top, self.scale = int(experts), int(top), float(scale)
+        self.score, self.normalise, self.act = score, bool(normalise), act
+        self.router = self.gate_up = self.down = None
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        n, E, F, H = self.name, self.experts, self.ffn_size, self.hidden_size
+        gu = tuple((f"{n}.e{e}.{m}", (F, H)) for e in range(E) for m in ("gate", "up"))
+        dn = tuple((f"{n}.e{e}.down", (H, F)) for e in range(E))
+        return [TensorSpec(f"{n}.router", (E, H), VECTOR, INIT_NORMAL),
+                TensorSpec(f"{n}.experts.gate_up", (E, 2 * F, H), MATRIX, INIT_NORMAL, pieces=gu,
+                           assemble=_stack_experts(E, (F, F)), split=_unstack_experts((F, F))),
+                TensorSpec(f"{n}.experts.down", (E, H, F), MATRIX, INIT_NORMAL, pieces=dn, assemble=_stack_experts(E, (H,)),
+                           split=_unstack_experts((H,)))]
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        n = self.name
+        self.router, self.gate_up, self.down = tensors[f"{n}.router"], tensors[f"{n}.experts.gate_up"], tensors[f"{n}.experts.down"]
+
+    def check_sizes(self) -> None:
+        if self.top > 64 or self.experts > 2048:
+            raise ValueError(f"{self.name}: the router takes at most 64 of at most 2048 experts")
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, add1=None, add2=None):
+        ids, wts = ops.moe_route(x, self.router, self.top, self.score, self.normalise, self.scale)
+        out = ops.moe_experts(x, self.gate_up, self.down, ids, wts, self.act)
+        if add1 is None and add2 is None:
+            return out
+        return ops.epilogue_(out, None, None, as_tensor(add1), as_tensor(add2))
+
+
 register_part("feed_forward", "dense", DenseFeedForward)
+register_part("feed_forward", "gated", GatedFeedForward)
+register_part("feed_forward", "routed", RoutedFeedForward)

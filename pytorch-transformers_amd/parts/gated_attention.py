@@ -1,0 +1,105 @@
+"""Attention with normed heads and an output gate.
+
+With h the mixer's input, H query heads on G key/value heads, queries and keys of ``key_dim`` elements and values of
+``value_dim``:
+
+    q = W_q h, k = W_k h, v = W_v h                       (no biases)
+    q, k <- head / sqrt(mean(head^2) + eps) * w_q | w_k    one weight [key_dim] for all heads, before the rotation
+    q, k <- rotated by position                            (``positions``: any rotation the kernels take)
+    v    <- head / sqrt(mean(head^2) + eps)                no weight; cached so
+    score(i, j) = q_i . k_j * scale, softmax over the keys j <= i that i sees:
+        all of them, those of i's own block of ``chunk`` positions (blocks counted from the sequence's start),
+        and / or the last ``window``
+    out = W_o (heads side by side * sigmoid(W_g h))
+
+The four products of h run as one (``Linear.stacked``).  The cache pages hold heads of ``frame`` >= max(key_dim,
+value_dim) elements, a size the attention kernels are built for; what lies past a head's own elements is zero, which
+changes neither scores nor sums.  Norms, angles, scores and the softmax are 32-bit.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Sequence
+
+import torch
+
+from .. import ops
+from ..engine.spec import INIT_ONE_NOISE, VECTOR, TensorSpec
+from .base import Part, StepContext, register_part
+from .linear import Linear
+from .positions import as_rotation
+
+
+def attention_frame(key_dim: int, value_dim: int) -> int:
+    """The head size of the cache pages for keys of ``key_dim`` and values of ``value_dim`` elements: the next size
+    the matrix-core attention is built for (multiples of 16 up to 128, and 256)."""
+    d = max(int(key_dim), int(value_dim))
+    return (d + 15) // 16 * 16 if d <= 128 else 256
+
+
+class GatedAttentionMixer(Part):
+    def __init__(self, name: str, hidden_size: int, num_heads: int, kv_heads: int, key_dim: int, value_dim: int,
+                 scale: float, eps: float, positions: Part, chunk: int = 0, window: int = 0, qk_norm: bool = True,
+                 v_norm: bool = True, gate: bool = True):
+        if num_heads % kv_heads:
+            raise ValueError(f"{name}: heads ({num_heads}) must be a multiple of kv heads ({kv_heads})")
+        self.name, self.hidden_size = name, int(hidden_size)
+        self.num_heads, self.kv_heads, self.key_dim, self.value_dim = int(num_heads), int(kv_heads), int(key_dim), int(value_dim)
+        self.scale, self.eps, self.positions = float(scale), float(eps), positions
+        self.chunk, self.window = int(chunk), int(window)
+        self.qk_norm, self.v_norm, self.gate = bool(qk_norm), bool(v_norm), bool(gate)
+        self.frame = attention_frame(key_dim, value_dim)
+        bare = lambda short, i, o: Linear(f"{name}.{short}", i, o, False, weight_name=f"{name}.{short}")
+        self.q = bare("q", hidden_size, self.num_heads * self.key_dim)
+        self.k = bare("k", hidden_size, self.kv_heads * self.key_dim)
+        self.v = bare("v", hidden_size, self.kv_heads * self.value_dim)
+        self.g = bare("g", hidden_size, self.num_heads * self.value_dim) if self.gate else None
+        self.out = bare("o", self.num_heads * self.value_dim, hidden_size)
+        self.q_w = self.k_w = None
+        self.inp: Optional[Linear] = None
+
+    def children(self) -> Sequence[Part]:
+        return tuple(p for p in (self.q, self.k, self.v, self.g, self.out, self.positions) if p is not None)
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        if not self.qk_norm:
+            return []
+        return [TensorSpec(f"{self.name}.q.norm", (self.key_dim,), VECTOR, INIT_ONE_NOISE),
+                TensorSpec(f"{self.name}.k.norm", (self.key_dim,), VECTOR, INIT_ONE_NOISE)]
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        if self.qk_norm:
+            self.q_w, self.k_w = tensors[f"{self.name}.q.norm"], tensors[f"{self.name}.k.norm"]
+
+    def after_load(self) -> None:
+        self.inp = Linear.stacked(f"{self.name}.qkvg", [p for p in (self.q, self.k, self.v, self.g) if p is not None])
+
+    def check_sizes(self) -> None:
+        rot = as_rotation(self.positions.rotation())
+        problem = ops.attention_sizes_problem(self.num_heads, self.kv_heads, self.frame, False)
+        if problem is None and max(self.key_dim, self.value_dim) > 256:
+            problem = f"heads of {max(self.key_dim, self.value_dim)} elements are more than the 256 the kernels take"
+        if problem is None and rot is not None:
+            problem = ops.rotation_problem(self.key_dim, rot.rotary_dim, rot.pairing)
+        if problem is None and (self.chunk < 0 or self.window < 0):
+            problem = "chunk and window are 0 (none) or positive"
+        if problem is not None:
+            raise ValueError(f"{self.name}: {problem}")
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, call, residual: Optional[torch.Tensor] = None):
+        k_pool, v_pool = ctx.cache.kv_layer(call.cache_group, call.cache_layer)
+        table = ctx.block_tables[call.cache_group]
+        H, G, dk, dv = self.num_heads, self.kv_heads, self.key_dim, self.value_dim
+        proj = self.inp(x)
+        at = [0, H * dk, (H + G) * dk, (H + G) * dk + G * dv]
+        q = ops.head_norm_rope_cache(proj[:, at[0]:at[1]], proj[:, at[1]:at[2]], proj[:, at[2]:at[3]], self.q_w, self.k_w,
+                                     self.eps, self.v_norm, as_rotation(self.positions.rotation()), ctx, table, k_pool,
+                                     v_pool, H, G, dk, dv, write_cache=call.write_cache)
+        o = ops.attention(q, k_pool, v_pool, table, ctx, None, self.scale, self.window, chunk=self.chunk)
+        if self.gate:
+            o = ops.gated_heads(o, self.frame, proj[:, at[3]:], H, dv, x.dtype)
+        elif self.frame != dv:
+            o = o.view(-1, H, self.frame)[:, :, :dv].reshape(-1, H * dv)
+        return self.out(o, add1=residual)
+
+
+register_part("mixer", "gated_attention", GatedAttentionMixer)

@@ -115,10 +115,16 @@ class RotaryPositions(NoPositions):
         self.rotary_dim = None if rotary_dim is None else int(rotary_dim)
         self.pairing = pairing
         if self.rotary_dim is not None:
-            if inv_freq is not None or dynamic_factor is not None:
-                raise ValueError("a rotation of part of a head goes with the default frequencies only")
+            if dynamic_factor is not None:
+                raise ValueError("a rotation of part of a head goes with frequencies that are fixed")
             if self.rotary_dim < 2 or self.rotary_dim % 2 or self.rotary_dim > head_dim:
                 raise ValueError(f"rotary_dim must be even, from 2 up to the head size {head_dim}; got {rotary_dim}")
+        if self.rotary_dim is not None and inv_freq is not None:
+            if tuple(inv_freq.shape) != (self.rotary_dim // 2,):  # a table of its own for the rotated part
+                raise ValueError(f"a frequency table for {self.rotary_dim} rotated elements has {self.rotary_dim // 2} "
+                                 f"entries, got {tuple(inv_freq.shape)}")
+            inv = inv_freq.to(torch.float32)
+        elif self.rotary_dim is not None:
             # (the powers taken in 64-bit and rounded once: a frequency is multiplied by positions in the thousands)
             inv = (1.0 / (self.theta ** (torch.arange(0, self.rotary_dim, 2, dtype=torch.float64) / self.rotary_dim))).float()
             if self.scaling_factor != 1.0:
@@ -181,6 +187,24 @@ def yarn_frequencies(head_dim: int, theta: float, factor: float, max_position_em
     turns_per_pos = theta ** (torch.arange(0, head_dim, 2).float() / head_dim)
     inv = (1.0 / (factor * turns_per_pos)) * (1 - keep) + (1.0 / turns_per_pos) * keep
     return inv, scale
+
+
+def yarn_ramp_frequencies(rotary_dim: int, base: float, factor: float, original: float, fast: float = 32.0,
+                          slow: float = 1.0):
+    """Frequencies ``f_i = base^(-2i / rotary_dim)`` stretched where they turn seldom within ``original`` positions:
+    with ``n(t) = rotary_dim * ln(original / (2 pi t)) / (2 ln base)`` the pair index whose frequency makes t turns
+    there, ``lo = max(floor(n(fast)), 0)``, ``hi = min(ceil(n(slow)), rotary_dim - 1)`` and the ramp ``r_i = clamp((i -
+    lo) / max(hi - lo, 0.001), 0, 1)``, the frequency is ``f_i / factor * r_i + f_i * (1 - r_i)``, and cosines and
+    sines are multiplied by ``0.1 ln(factor) + 1``.  Evaluated in 64-bit and rounded once; returns (table, that
+    factor)."""
+    half = rotary_dim // 2
+    pair_with_turns = lambda t: rotary_dim * math.log(original / (2.0 * math.pi * t)) / (2.0 * math.log(base))
+    lo = max(math.floor(pair_with_turns(fast)), 0)
+    hi = min(math.ceil(pair_with_turns(slow)), rotary_dim - 1)
+    i = torch.arange(half, dtype=torch.float64)
+    f = float(base) ** (-2.0 * i / rotary_dim)
+    ramp = torch.clamp((i - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+    return (f / float(factor) * ramp + f * (1.0 - ramp)).float(), 0.1 * math.log(float(factor)) + 1.0
 
 
 def llama3_frequencies(head_dim: int, theta: float, factor: float, low_freq_factor: float, high_freq_factor: float,

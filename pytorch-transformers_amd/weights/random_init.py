@@ -75,7 +75,12 @@ def write_random_model(folder: str, config, seed: int, *, std: Optional[float] =
     _, builder = lookup(config.model_type)
     spec = builder(config)
     std = float(getattr(config, "initializer_range", 0.02) if std is None else std)
-    tensors = random_tensors(spec.tensor_specs(), seed, std, noise=noise, store_dtype=store_dtype)
+    specs = spec.tensor_specs()
+    tensors = random_tensors(specs, seed, std, noise=noise, store_dtype=store_dtype)
+    for s in specs:  # a tensor that the design's files hold in pieces is written so
+        if s.split is not None and s.name in tensors:
+            for (name, _), piece in zip(s.pieces, s.split(tensors.pop(s.name))):
+                tensors[name] = piece.contiguous()
     os.makedirs(folder, exist_ok=True)
     config.save_pretrained(folder)
     save_weights(folder, tensors, shards=shards)
