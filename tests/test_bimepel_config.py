@@ -1,0 +1,81 @@
+"""The Bimepel design's configuration, run order, tensor names and cache groups (no GPU)."""
+import pytest
+
+from pytorch_transformers_amd.config import AutoConfig, ConfigError
+from pytorch_transformers_amd.config.registry import lookup
+
+
+def _attn(**over):
+    m = {"heads": 4, "kv_heads": 2, "dim": 24, "vdim": 20, "scale": 0.2, "rot": {"base": 1e4, "dims": 8}, "mask": {"size": 40}}
+    m.update(over)
+    return {"type": "attention", "mixer": m, "mlp": {"kind": "dense", "ff": 32, "limit": 1.5}}
+
+
+def _lin(**over):
+    m = {"heads": 2, "dim": 8, "vdim": 12, "decay": [0.5, 0.9]}
+    m.update(over)
+    return {"type": "lightning", "mixer": m,
+            "mlp": {"kind": "moe", "expert": {"ff": 8}, "router": {"experts": 3, "top": 2, "scale": 1.0}}}
+
+
+def _cfg(layers, **more):
+    return dict({"architecture": "Bimepel", "vocab": 50, "width": 32, "norm": {"eps": 1e-5}, "layers": layers}, **more)
+
+
+def test_the_architecture_key_chooses_the_design():
+    cfg = AutoConfig.from_dict(_cfg([_attn(), _lin()]))
+    assert type(cfg).__name__ == "BimepelConfig" and cfg.model_type == "bimepel" and cfg.vocab_size == 50
+    assert cfg.run_order() == [0, 1]
+
+
+def test_a_loop_repeats_its_layers_in_a_row():
+    cfg = AutoConfig.from_dict(_cfg([_attn(), _lin(), _attn(), _lin()], loop={"start": 1, "stop": 3, "times": 3}))
+    assert cfg.run_order() == [0, 1, 2, 1, 2, 1, 2, 3]
+    assert AutoConfig.from_dict(_cfg([_attn(), _lin()], loop={"start": 0, "stop": 2, "times": 1})).run_order() == [0, 1]
+    assert AutoConfig.from_dict(_cfg([_attn(), _lin()], loop={"start": 1, "stop": 1, "times": 4})).run_order() == [0, 1]
+
+
+@pytest.mark.parametrize("layers,more,word", [
+    ([dict(_attn(), type="conv")], {}, "type"),
+    ([_attn(kv_heads=3)], {}, "multiple"),
+    ([_attn(rot={"base": 1e4, "dims": 26})], {}, "dims"),
+    ([_attn(rot={"base": 1e4, "dims": 7})], {}, "dims"),
+    ([_attn(mask={"size": 0})], {}, "size"),
+    ([_lin(decay=[0.5])], {}, "decay"),
+    ([dict(_attn(), mlp={"kind": "conv"})], {}, "kind"),
+    ([dict(_attn(), mlp={"kind": "dense", "ff": 8})], {}, "limit"),
+    ([dict(_lin(), mlp={"kind": "moe", "expert": {"ff": 8}, "router": {"experts": 2, "top": 3, "scale": 1.0}})], {}, "top"),
+    ([_attn()], {"loop": {"start": 0, "stop": 2, "times": 2}}, "loop"),
+    ([_attn()], {"loop": {"start": 0, "stop": 1, "times": 0}}, "loop"),
+    ([], {}, "layers"),
+])
+def test_what_cannot_run_is_refused_by_name(layers, more, word):
+    with pytest.raises(ConfigError, match=word):
+        AutoConfig.from_dict(_cfg(layers, **more))
+
+
+def test_tensor_names_and_storage_of_every_pass():
+    layers = [_attn(), _lin(), dict(_attn(kv_heads=1, dim=16, vdim=32, rot=None, mask=None), mlp=None), _lin(heads=1, decay=[0.7])]
+    cfg = AutoConfig.from_dict(_cfg(layers, loop={"start": 0, "stop": 3, "times": 2}))
+    spec = lookup(cfg.model_type)[1](cfg)
+    spec.validate()
+    names = set()
+    for s in spec.tensor_specs():
+        names |= {n for n, _ in s.pieces} if s.pieces else {s.name}
+    assert {"embed", "final.norm", "l0.norm1", "l0.norm2", "l0.shift", "l0.mix.q", "l0.mix.k", "l0.mix.v", "l0.mix.g", "l0.mix.o",
+            "l0.mix.q.norm", "l0.mix.k.norm", "l0.mlp.gate", "l0.mlp.up", "l0.mlp.down", "l1.mix.norm", "l1.mlp.router",
+            "l1.mlp.e0.gate", "l1.mlp.e2.down", "l2.mix.o", "l3.mlp.e1.up"} <= names
+    assert "l2.norm2" not in names and not any(n.startswith("l2.mlp") for n in names)
+    shapes = {s.name: s.shape for s in spec.tensor_specs()}
+    assert shapes["l0.mix.q"] == (96, 32) and shapes["l0.mix.k"] == (48, 32) and shapes["l0.mix.v"] == (40, 32)
+    assert shapes["l0.mix.g"] == (80, 32) and shapes["l0.mix.o"] == (32, 80) and shapes["l1.mix.norm"] == (24,)
+    # seven passes: each its own row of the shift table and its own layer of its mixer's storage
+    assert [c.block for c in spec.order] == [0, 1, 2, 0, 1, 2, 3]
+    assert sorted(c.also("shift") for c in spec.order) == [("shift", i) for i in range(7)]
+    assert len({(c.cache_group, c.cache_layer) for c in spec.order}) == 7
+    groups = {g.name: g for g in spec.cache_groups}
+    assert groups["shift"].num_layers == 7 and groups["shift"].state_shape == (32,)
+    kv = sorted((g.kv_heads, g.head_dim, g.num_layers) for g in groups.values() if g.kind == "full")
+    assert kv == [(1, 32, 2), (2, 32, 2)]
+    states = sorted((g.state_shape, g.num_layers) for g in groups.values() if g.kind == "state" and g.name != "shift")
+    assert states == [((96,), 1), ((192,), 2)]
