@@ -393,6 +393,49 @@ def pavodra_config(size, layers, vocab=32768):
                          residual_mult=0.3, logit_scale=1.0, initializer_range=0.02)
 
 
+# ---- the Bimepel design beside the same Falcon model (--design bimepel) --------------------------------------------------
+BIMEPEL_SIZES = {
+    # width; the dense feed-forward's size (three matrices: two thirds of Falcon's feed-forward for as many weights);
+    # attention heads of 128 on 8 KV heads, half of a head rotated, blocks of 8,192 positions; linear attention heads
+    # of 128 x 128; 16 experts of which a token uses 2, which together are as large as the dense feed-forward
+    "2k": dict(width=2048, ff=5504, heads=16, lin_heads=16, expert_ff=2752),
+    "4k": dict(width=4096, ff=10880, heads=32, lin_heads=32, expert_ff=5440),
+}
+BIMEPEL_KERNEL_LABELS = {
+    "pta_shift_norm": "residual sum into the 32-bit stream, two RMS norms, token shift",
+    "pta_wide_sum": "residual sum in front of the final norm",
+    "pta_head_norm_rope_cache": "query / key / value norms, rotation, cache write",
+    "pta_gated_heads": "output gate (linear attention: with its norm)",
+    "pta_glu": "the dense feed-forward's clamped gate",
+    "pta_decay_scan": "linear attention's recurrence",
+    "pta_moe_route": "router: scores, the experts taken and their weights",
+    "pta_moe_up": "experts' gate and up products, a row of W per wave (few tokens)",
+    "pta_moe_down": "experts' down products and weighted sum (few tokens)",
+    "pta_moe_sort": "(token, expert) pairs sorted by expert",
+    "pta_moe_grouped_up": "experts' gate and up products on the matrix cores, tiles of one expert's tokens",
+    "pta_moe_grouped_down": "experts' down products on the matrix cores",
+    "pta_moe_combine": "weighted sum of a token's experts",
+}
+
+
+def bimepel_config(size, layers, vocab=32768):
+    """Four layers (attention + dense, linear attention + experts, attention + experts, linear attention + dense) of
+    which the middle two run ``layers - 2`` / 2 times: ``layers`` layer runs."""
+    from pytorch_transformers_amd import BimepelConfig
+
+    z = BIMEPEL_SIZES[size]
+    dense = {"kind": "dense", "ff": z["ff"], "limit": 7.0}
+    moe = {"kind": "moe", "expert": {"ff": z["expert_ff"]}, "router": {"experts": 16, "top": 2, "scale": 1.0}}
+    attn = {"heads": z["heads"], "kv_heads": 8, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "mask": {"size": 8192},
+            "rot": {"base": 10000.0, "dims": 64, "scaling": {"factor": 4.0, "original": 2048, "fast": 32.0, "slow": 1.0}}}
+    lin = {"heads": z["lin_heads"], "dim": 128, "vdim": 128,
+           "decay": [1.0 - 2.0 ** (-5.0 - 3.0 * h / max(1, z["lin_heads"] - 1)) for h in range(z["lin_heads"])]}
+    kinds = [{"type": "attention", "mixer": attn, "mlp": dense}, {"type": "lightning", "mixer": lin, "mlp": moe},
+             {"type": "attention", "mixer": attn, "mlp": moe}, {"type": "lightning", "mixer": lin, "mlp": dense}]
+    return BimepelConfig(vocab=vocab, width=z["width"], layers=kinds, loop={"start": 1, "stop": 3, "times": max(1, (layers - 2) // 2)},
+                         norm={"eps": 1e-6}, initializer_range=0.02)
+
+
 def falcon_like(size, layers, vocab=32768):
     """The closest model the library had: Falcon's new architecture at the same width, feed-forward, depth and
     vocabulary, heads of 128 in 8 groups."""
@@ -415,15 +458,18 @@ def design_record(args):
 
     ops.load_library()
     KERNEL_LABELS.update(PAVODRA_KERNEL_LABELS)
+    KERNEL_LABELS.update(BIMEPEL_KERNEL_LABELS)
+    design = args.design
+    design_config = pavodra_config if design == "pavodra" else bimepel_config
     gen_cfg = GenerationConfig(do_sample=False, eos_token_id=None)
     layers, T, ctx_len = args.layers or 6, args.prefill_tokens, args.prompt_len
-    out = {"design": "pavodra", "beside": "falcon (new architecture, 8 KV groups of head size 128)", "dtype": args.dtype,
+    out = {"design": design, "beside": "falcon (new architecture, 8 KV groups of head size 128)", "dtype": args.dtype,
            "layers": layers, "prefill_tokens": T, "decode_context": ctx_len, "data": "synthetic token ids, random weights",
            "sizes": {}}
     dtype = "bfloat16" if args.dtype == "bf16" else "float32"
     for size in args.design_sizes.split(","):
         rec = {}
-        for name, cfg in (("pavodra", pavodra_config(size, layers)), ("falcon", falcon_like(size, layers))):
+        for name, cfg in ((design, design_config(size, layers)), ("falcon", falcon_like(size, layers))):
             model = AutoModelForCausalLM.from_config(cfg, seed=0, dtype=dtype, device="cuda:0")
             r = {}
             pt = run_prefill(model, T)
@@ -442,6 +488,12 @@ def design_record(args):
                 if name == "pavodra":
                     row, heads, rank = 576, PAVODRA_SIZES[size]["heads"], 512
                     kv, fl = b * (ctx_len + 1) * row * 2, 2.0 * heads * (row + rank) * T * (T + 1) / 2
+                elif name == "bimepel":  # keys and values of a token's own block of positions only
+                    a = cfg.layers[0]["mixer"]
+                    block = a["mask"]["size"]
+                    kv = b * (ctx_len % block + 1) * a["kv_heads"] * (a["dim"] + a["vdim"]) * 2
+                    seen = sum(min(block, T - s0) * (min(block, T - s0) + 1) / 2 for s0 in range(0, T, block))
+                    fl = 2.0 * (a["dim"] + a["vdim"]) * a["heads"] * seen
                 else:
                     kv = b * (ctx_len + 1) * 2 * cfg.kv_heads * cfg.head_dim * 2
                     fl = 2.0 * cfg.head_dim * cfg.num_attention_heads * T * (T + 1)
@@ -469,7 +521,7 @@ def design_record(args):
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--design", default=None, choices=["pavodra"],
+    ap.add_argument("--design", default=None, choices=["pavodra", "bimepel"],
                     help="measure that design beside the closest Falcon model at equal layer sizes and print that record "
                          "instead of the default run's (--layers, --prefill-tokens, --prompt-len and --dtype apply)")
     ap.add_argument("--design-sizes", default="2k,4k", help="with --design: which of the layer sizes 2k, 4k")

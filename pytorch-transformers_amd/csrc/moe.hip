@@ -20,7 +20,15 @@
 template <typename T>
 __device__ __forceinline__ float wave_dot(const T* __restrict__ w, const float* __restrict__ x_s, int K, int lane) {
     float acc = 0.f;
-    if (sizeof(T) == 2 && (K & 7) == 0 && ((uintptr_t)w & 15) == 0) {
+    if (sizeof(T) == 4 && (K & 3) == 0 && ((uintptr_t)w & 15) == 0) {
+#pragma unroll 4
+        for (int k = lane * 4; k < K; k += PTA_WAVE * 4) {
+            const float4 f = *reinterpret_cast<const float4*>((const float*)w + k);
+            const float4 xv = *reinterpret_cast<const float4*>(x_s + k);
+            acc += f.x * xv.x + f.y * xv.y + f.z * xv.z + f.w * xv.w;
+        }
+    } else if (sizeof(T) == 2 && (K & 7) == 0 && ((uintptr_t)w & 15) == 0) {
+#pragma unroll 2
         for (int k = lane * 8; k < K; k += PTA_WAVE * 8) {
             float f[8];
             unpack8(*reinterpret_cast<const uint4*>((const bf16_t*)w + k), f);
@@ -172,4 +180,200 @@ extern "C" int pta_moe_down(void* out, const void* act_in, const void* down, con
     else
         hipLaunchKernelGGL(moe_down_kernel<bf16_t>, grid, dim3(256), (size_t)top * F * 4, s, (bf16_t*)out, (const bf16_t*)act_in, (const bf16_t*)down, ids, wts, H, F, top);
     return pta_check_launch("moe_down");
+}
+
+// ---- steps of many tokens: tiles of one expert's tokens on the matrix cores --------------------------------------------
+// pta_moe_sort lays the (token, expert) pairs out by expert: every expert's pairs take a run of slots that starts at a
+// multiple of MOE_TILE, the slots between an expert's last pair and the next multiple hold -1.  tile_expert[t] is the
+// expert of slots t * MOE_TILE .. + MOE_TILE - 1 (-1: no such tile), slot_of_pair[p] where pair p went.  One workgroup;
+// the order of an expert's pairs among themselves is whatever the atomics give, and no result depends on it (a row's
+// products are the same sums wherever the row lies).
+#define MOE_TILE 64
+
+__global__ __launch_bounds__(1024) void moe_sort_kernel(int* __restrict__ sorted_pair, int* __restrict__ slot_of_pair,
+                                                        int* __restrict__ tile_expert, const int* __restrict__ ids, int pairs,
+                                                        int E, int slots, int tiles) {
+    extern __shared__ int sm_i[];
+    int* count = sm_i;          // [E]
+    int* start = sm_i + E;      // [E + 1], in slots
+    int* cursor = start + E + 1;  // [E]
+    for (int e = threadIdx.x; e < E; e += blockDim.x) { count[e] = 0; cursor[e] = 0; }
+    for (int i = threadIdx.x; i < slots; i += blockDim.x) sorted_pair[i] = -1;
+    for (int t = threadIdx.x; t < tiles; t += blockDim.x) tile_expert[t] = -1;
+    __syncthreads();
+    for (int p = threadIdx.x; p < pairs; p += blockDim.x) atomicAdd(&count[ids[p]], 1);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int at = 0;
+        for (int e = 0; e < E; ++e) {
+            start[e] = at;
+            at += (count[e] + MOE_TILE - 1) / MOE_TILE * MOE_TILE;
+        }
+        start[E] = at;
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < E; e += blockDim.x)
+        for (int t = start[e] / MOE_TILE; t < start[e + 1] / MOE_TILE; ++t) tile_expert[t] = e;
+    for (int p = threadIdx.x; p < pairs; p += blockDim.x) {
+        const int e = ids[p];
+        const int slot = start[e] + atomicAdd(&cursor[e], 1);
+        sorted_pair[slot] = p;
+        slot_of_pair[p] = slot;
+    }
+}
+
+typedef __bf16 moe_bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float moe_f32x4_t __attribute__((ext_vector_type(4)));
+union MoeFrag { uint4 u; moe_bf16x8_t v; };
+
+__device__ __forceinline__ uint32_t moe_pack2(float lo, float hi) {
+    return (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
+}
+
+// act_sorted[slot, f] = act(G_e x) * (U_e x) for the slot's pair (token, e).  A workgroup of four waves owns a tile of
+// MOE_TILE slots and 64 rows f of its expert; a wave owns sixteen rows of the gate and the same sixteen of the up
+// matrix against all four groups of sixteen tokens: W rows are the A operand (sixteen bytes of a row per lane), x rows
+// the B operand, both straight from memory (the four waves read the same x rows, which the caches hold).
+__global__ __launch_bounds__(256) void moe_grouped_up_kernel(bf16_t* __restrict__ act_sorted, const bf16_t* __restrict__ x,
+                                                             long x_ld, const bf16_t* __restrict__ gate_up,
+                                                             const int* __restrict__ sorted_pair,
+                                                             const int* __restrict__ tile_expert, int H, int F, int top,
+                                                             int act) {
+    const int tile = blockIdx.x, e = tile_expert[tile];
+    if (e < 0) return;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, gq = lane >> 4;
+    const int f0 = blockIdx.y * 64 + wave * 16;
+    if (f0 >= F) return;
+    const int fr = min(f0 + c, F - 1);
+    const bf16_t* G = gate_up + ((long)e * 2 * F + fr) * H + gq * 8;
+    const bf16_t* U = G + (long)F * H;
+    const bf16_t* xr[4];
+#pragma unroll
+    for (int tt = 0; tt < 4; ++tt) {
+        const int pair = sorted_pair[tile * MOE_TILE + tt * 16 + c];
+        xr[tt] = x + (long)(pair < 0 ? 0 : pair / top) * x_ld + gq * 8;
+    }
+    moe_f32x4_t ag[4], au[4];
+#pragma unroll
+    for (int tt = 0; tt < 4; ++tt) { ag[tt] = moe_f32x4_t{0.f, 0.f, 0.f, 0.f}; au[tt] = moe_f32x4_t{0.f, 0.f, 0.f, 0.f}; }
+    for (int k = 0; k < H; k += 32) {
+        MoeFrag wg, wu, xb[4];
+        wg.u = *reinterpret_cast<const uint4*>(G + k);
+        wu.u = *reinterpret_cast<const uint4*>(U + k);
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt) xb[tt].u = *reinterpret_cast<const uint4*>(xr[tt] + k);
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt) {
+            ag[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wg.v, xb[tt].v, ag[tt], 0, 0, 0);
+            au[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wu.v, xb[tt].v, au[tt], 0, 0, 0);
+        }
+    }
+    // acc[j] is row f0 + 4 gq + j of the token in column c
+#pragma unroll
+    for (int tt = 0; tt < 4; ++tt) {
+        const long slot = (long)tile * MOE_TILE + tt * 16 + c;
+        float y[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) y[j] = apply_act(round_to_bf16(ag[tt][j]), act) * round_to_bf16(au[tt][j]);
+        bf16_t* dst = act_sorted + slot * F + f0 + 4 * gq;
+        if (f0 + 4 * gq + 3 < F) {
+            uint2 w2;
+            w2.x = moe_pack2(y[0], y[1]);
+            w2.y = moe_pack2(y[2], y[3]);
+            *reinterpret_cast<uint2*>(dst) = w2;
+        } else {
+            for (int j = 0; j < 4; ++j)
+                if (f0 + 4 * gq + j < F) dst[j] = f32_to_bf16_bits(y[j]);
+        }
+    }
+}
+
+// y_sorted[slot, n] = D_e act_sorted[slot]: a wave owns two groups of sixteen rows n of the expert's down matrix against
+// the tile's four groups of sixteen slots; a workgroup 128 rows
+__global__ __launch_bounds__(256) void moe_grouped_down_kernel(bf16_t* __restrict__ y_sorted, const bf16_t* __restrict__ act_sorted,
+                                                               const bf16_t* __restrict__ down,
+                                                               const int* __restrict__ tile_expert, int H, int F) {
+    const int tile = blockIdx.x, e = tile_expert[tile];
+    if (e < 0) return;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, gq = lane >> 4;
+    const int n0 = blockIdx.y * 128 + wave * 32;
+    if (n0 >= H) return;
+    const bf16_t* D0 = down + ((long)e * H + min(n0 + c, H - 1)) * F + gq * 8;
+    const bf16_t* D1 = down + ((long)e * H + min(n0 + 16 + c, H - 1)) * F + gq * 8;
+    const bf16_t* ar = act_sorted + ((long)tile * MOE_TILE + c) * F + gq * 8;
+    moe_f32x4_t a0[4], a1[4];
+#pragma unroll
+    for (int tt = 0; tt < 4; ++tt) { a0[tt] = moe_f32x4_t{0.f, 0.f, 0.f, 0.f}; a1[tt] = moe_f32x4_t{0.f, 0.f, 0.f, 0.f}; }
+    for (int k = 0; k < F; k += 32) {
+        MoeFrag w0, w1, xb[4];
+        w0.u = *reinterpret_cast<const uint4*>(D0 + k);
+        w1.u = *reinterpret_cast<const uint4*>(D1 + k);
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt) xb[tt].u = *reinterpret_cast<const uint4*>(ar + (long)tt * 16 * F + k);
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt) {
+            a0[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0.v, xb[tt].v, a0[tt], 0, 0, 0);
+            a1[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1.v, xb[tt].v, a1[tt], 0, 0, 0);
+        }
+    }
+#pragma unroll
+    for (int tt = 0; tt < 4; ++tt) {
+        const long slot = (long)tile * MOE_TILE + tt * 16 + c;
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            const moe_f32x4_t& a = half ? a1[tt] : a0[tt];
+            const int n = n0 + half * 16 + 4 * gq;
+            bf16_t* dst = y_sorted + slot * H + n;
+            if (n + 3 < H) {
+                uint2 w2;
+                w2.x = moe_pack2(a[0], a[1]);
+                w2.y = moe_pack2(a[2], a[3]);
+                *reinterpret_cast<uint2*>(dst) = w2;
+            } else {
+                for (int j = 0; j < 4; ++j)
+                    if (n + j < H) dst[j] = f32_to_bf16_bits(a[j]);
+            }
+        }
+    }
+}
+
+// out[m, n] = sum_k wts[m, k] * y_sorted[slot_of_pair[m * top + k], n], in the order the experts were taken
+__global__ void moe_combine_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ y_sorted,
+                                   const int* __restrict__ slot_of_pair, const float* __restrict__ wts, int H, int top) {
+    const int m = blockIdx.x;
+    for (int n = threadIdx.x; n < H; n += blockDim.x) {
+        float acc = 0.f;
+        for (int k = 0; k < top; ++k)
+            acc += wts[(long)m * top + k] * bf16_bits_to_f32(y_sorted[(long)slot_of_pair[(long)m * top + k] * H + n]);
+        out[(long)m * H + n] = f32_to_bf16_bits(acc);
+    }
+}
+
+extern "C" int pta_moe_grouped_slots(int pairs, int E) { return (pairs + E * (MOE_TILE - 1) + MOE_TILE - 1) / MOE_TILE * MOE_TILE; }
+
+// bfloat16 only; H and F multiples of 32.  sorted_pair [slots], slot_of_pair [M * top], tile_expert [slots / 64],
+// act_sorted [slots, F], y_sorted [slots, H] are the caller's scratch (slots = pta_moe_grouped_slots(M * top, E)).
+extern "C" int pta_moe_grouped(void* out, const void* x, long x_ld, const void* gate_up, const void* down, const int* ids,
+                               const float* wts, int* sorted_pair, int* slot_of_pair, int* tile_expert, void* act_sorted,
+                               void* y_sorted, int M, int H, int F, int E, int top, int act, void* stream) {
+    PTA_REQUIRE(M > 0 && H > 0 && F > 0 && E > 0 && top > 0, "moe_grouped: sizes must be positive");
+    PTA_REQUIRE(H % 32 == 0 && F % 32 == 0 && x_ld % 8 == 0, "moe_grouped: features (%d) and expert size (%d) must be multiples of 32", H, F);
+    PTA_REQUIRE(out && x && gate_up && down && ids && wts && sorted_pair && slot_of_pair && tile_expert && act_sorted && y_sorted,
+                "moe_grouped: null pointer");
+    PTA_REQUIRE((((uintptr_t)x | (uintptr_t)gate_up | (uintptr_t)down | (uintptr_t)act_sorted | (uintptr_t)y_sorted) % 16) == 0,
+                "moe_grouped: matrices must be aligned to sixteen bytes");
+    PTA_REQUIRE(pta_act_known(act), "moe_grouped: unknown activation %d", act);
+    PTA_REQUIRE((size_t)(3 * E + 1) * 4 <= 64 * 1024, "moe_grouped: %d experts are more than the sort holds", E);
+    const long pairs = (long)M * top;
+    const int slots = pta_moe_grouped_slots((int)pairs, E), tiles = slots / MOE_TILE;
+    PTA_REQUIRE(pairs < (1L << 30) && tiles <= 2147483647 / 64, "moe_grouped: too many pairs");
+    hipStream_t s = (hipStream_t)stream;
+    hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), (size_t)(3 * E + 1) * 4, s, sorted_pair, slot_of_pair, tile_expert,
+                       ids, (int)pairs, E, slots, tiles);
+    hipLaunchKernelGGL(moe_grouped_up_kernel, dim3(tiles, (F + 63) / 64), dim3(256), 0, s, (bf16_t*)act_sorted, (const bf16_t*)x,
+                       x_ld, (const bf16_t*)gate_up, sorted_pair, tile_expert, H, F, top, act);
+    hipLaunchKernelGGL(moe_grouped_down_kernel, dim3(tiles, (H + 127) / 128), dim3(256), 0, s, (bf16_t*)y_sorted,
+                       (const bf16_t*)act_sorted, (const bf16_t*)down, tile_expert, H, F);
+    hipLaunchKernelGGL(moe_combine_kernel, dim3(M), dim3(256), 0, s, (bf16_t*)out, (const bf16_t*)y_sorted, slot_of_pair, wts, H, top);
+    return pta_check_launch("moe_grouped");
 }

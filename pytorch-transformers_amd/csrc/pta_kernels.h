@@ -315,6 +315,10 @@ int pta_moe_up(void* act_out, const void* h, long h_ld, const void* gate_up, con
                int act, int dtype, void* stream);
 int pta_moe_down(void* out, const void* act_in, const void* down, const int* ids, const float* wts, int M, int H, int F,
                  int top, int dtype, void* stream);
+int pta_moe_grouped_slots(int pairs, int E);
+int pta_moe_grouped(void* out, const void* x, long x_ld, const void* gate_up, const void* down, const int* ids,
+                    const float* wts, int* sorted_pair, int* slot_of_pair, int* tile_expert, void* act_sorted, void* y_sorted,
+                    int M, int H, int F, int E, int top, int act, void* stream);
 
 #ifdef __cplusplus
 }

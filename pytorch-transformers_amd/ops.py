@@ -194,6 +194,36 @@ def _entry_cost(name: str, a) -> tuple:
         return (H * K * O * (4.0 if a[13] == F32 else 2.0) + M * H * (K + O) * 4.0, 2.0 * M * H * K * O)
     if name == "pta_latent_prep":
         return (float(a[11]) * val(3) * (4.0 if a[17] == F32 else 2.0), 0.0)
+    el = lambda code: 4.0 if code == F32 else 2.0
+    if name == "pta_shift_norm":  # the stream in and out (32-bit), the terms in, the two norms out
+        M, H, e = float(a[16]), float(a[17]), el(a[20])
+        return (M * H * (4.0 + given(2) * 4.0 + (given(4) + given(5)) * e + (1.0 + given(1)) * e), 0.0)
+    if name == "pta_wide_sum":
+        return (val(4) * (8.0 + (1.0 + given(3)) * el(a[5])), 0.0)
+    if name == "pta_head_norm_rope_cache":  # the heads in, the queries' frames and the pages' rows out
+        M, e = float(a[16]), el(a[23])
+        return (M * e * ((a[17] + a[18]) * (a[19] + a[21]) + a[18] * (a[20] + a[21])), 0.0)
+    if name == "pta_gated_heads":
+        M, N, e = float(a[9]), float(a[10] * a[11]), el(a[12])
+        return (M * N * ((4.0 if a[2] else e) + 2 * e), 0.0)
+    if name == "pta_glu":
+        return (float(a[4]) * a[5] * 3 * el(a[9]), 0.0)
+    if name == "pta_decay_scan":  # q, k, v in, o out in 32-bit; two multiply-adds per state element and token
+        M, heads, P, N, e = float(timing_hint.get("rows", 0)), a[12], a[13], a[14], el(a[18])
+        return (M * heads * ((2 * N + P) * e + P * 4.0), 4.0 * M * heads * N * P)
+    if name == "pta_moe_route":
+        return (float(a[5]) * a[6] * el(a[12]) + float(a[6]) * a[7] * 4.0, 2.0 * a[5] * a[6] * a[7])
+    if name == "pta_moe_up":  # at most every (token, expert) pair's matrices once, and no more than all experts'
+        M, H, Fe, top, e = float(a[5]), a[6], a[7], a[8], el(a[10])
+        pairs = min(M * top, float(timing_hint.get("experts", M * top)))
+        return (pairs * 2 * Fe * H * e, 4.0 * M * top * Fe * H)
+    if name == "pta_moe_down":
+        M, H, Fe, top, e = float(a[5]), a[6], a[7], a[8], el(a[9])
+        pairs = min(M * top, float(timing_hint.get("experts", M * top)))
+        return (pairs * Fe * H * e, 2.0 * M * top * Fe * H)
+    if name == "pta_moe_grouped":  # every expert's three matrices once; the arithmetic of the pairs
+        M, H, Fe, E, top = float(a[12]), a[13], a[14], a[15], a[16]
+        return (min(E, M * top) * 3.0 * Fe * H * 2.0, 6.0 * M * top * Fe * H)
     return (0.0, 0.0)
 
 
@@ -1492,7 +1522,7 @@ def glu(gate: torch.Tensor, up: torch.Tensor, kind: str = "silu", alpha: float =
 
 
 # ---- linear attention with a decay per head -------------------------------------------------------------------------
-DECAY_SCAN_CHUNK_TOKENS = 128  # a sequence that brings more than twice as many tokens is cut into chunks that run side by side
+DECAY_SCAN_CHUNK_TOKENS = 64  # a sequence that brings more than twice as many tokens is cut into chunks that run side by side
 
 
 def decay_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Tensor, state: torch.Tensor, cu_tokens,
@@ -1511,6 +1541,7 @@ def decay_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.T
     _need(cu_tokens, "cu_tokens", torch.int32, (n + 1,))
     state_ld = _need_state(state, heads * key_dim * value_dim)
     y = torch.empty((M, heads * value_dim), dtype=torch.float32, device=q.device)
+    timing_hint["rows"] = M
     chunk, chunks = DECAY_SCAN_CHUNK_TOKENS, 1
     if max_new > 2 * chunk:
         chunks = (int(max_new) + chunk - 1) // chunk
@@ -1544,6 +1575,9 @@ def moe_route(h: torch.Tensor, router: torch.Tensor, top: int, score: str = "sig
     return ids, wts
 
 
+MOE_GROUPED_FROM_ROWS = 16  # steps of more tokens run their experts on the matrix cores (bfloat16)
+
+
 def moe_experts(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor,
                 act: str = "silu") -> torch.Tensor:
     """``sum_k wts[m, k] * down[e] (act(gate[e] h) * (up[e] h))`` with ``e = ids[m, k]``: ``gate_up`` ``[experts, 2 F,
@@ -1557,8 +1591,20 @@ def moe_experts(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, ids:
     _need(ids, "ids", torch.int32, (M, top))
     _need(wts, "wts", torch.float32, (M, top))
     ld = _rows_of(h, "h", H, h.dtype)
-    act_buf = torch.empty((M * top, F), dtype=h.dtype, device=h.device)
     out = torch.empty((M, H), dtype=h.dtype, device=h.device)
+    timing_hint["experts"] = E
+    if (h.dtype == torch.bfloat16 and M > MOE_GROUPED_FROM_ROWS and H % 32 == 0 and F % 32 == 0 and ld % 8 == 0
+            and h.data_ptr() % 16 == 0):
+        # many tokens: the pairs sorted by expert, tiles of one expert's tokens on the matrix cores
+        slots = load_library().pta_moe_grouped_slots(M * top, E)
+        ints = torch.empty(slots + M * top + slots // 64, dtype=torch.int32, device=h.device)
+        act_sorted = torch.empty((slots, F), dtype=h.dtype, device=h.device)
+        y_sorted = torch.empty((slots, H), dtype=h.dtype, device=h.device)
+        _call("pta_moe_grouped", _ptr(out), _ptr(h), ctypes.c_long(ld), _ptr(gate_up), _ptr(down), _ptr(ids), _ptr(wts),
+              _ptr(ints[:slots]), _ptr(ints[slots:slots + M * top]), _ptr(ints[slots + M * top:]), _ptr(act_sorted),
+              _ptr(y_sorted), M, H, F, E, top, ACT_CODES[act], _stream())
+        return out
+    act_buf = torch.empty((M * top, F), dtype=h.dtype, device=h.device)
     if M:
         _call("pta_moe_up", _ptr(act_buf), _ptr(h), ctypes.c_long(ld), _ptr(gate_up), _ptr(ids), M, H, F, top,
               ACT_CODES[act], dtype_code(h.dtype), _stream())

@@ -239,8 +239,15 @@ class ShiftedParallelBlock(Part):
         state = ctx.cache.state_layer(group, layer)
         stream, a, m = ops.shift_norm(base, terms, self.norm_mixer.weight, None if self.norm_ffn is None else self.norm_ffn.weight,
                                       self.mu, self.norm_mixer.eps, state, ctx, ctx.dtype)
-        mixed = self.mixer.forward(a, ctx, call)
-        ff = self.feed_forward.forward(m, ctx) if self.feed_forward is not None else None
+        kw_mixer, kw_ffn = {}, {}
+        # both branches start with a product of a norm of x: one launch for the two in small steps
+        if hasattr(self.mixer, "input_projection") and hasattr(self.feed_forward, "input_projection"):
+            (lin_a, kw_a), (lin_m, kw_m) = self.mixer.input_projection(), self.feed_forward.input_projection()
+            both = Linear.pair(lin_a, a, kw_a, lin_m, m, kw_m) if lin_a is not None and lin_m is not None else None
+            if both is not None:
+                kw_mixer["projected"], kw_ffn["projected"] = both
+        mixed = self.mixer.forward(a, ctx, call, **kw_mixer)
+        ff = self.feed_forward.forward(m, ctx, **kw_ffn) if self.feed_forward is not None else None
         return WideSum(stream, [mixed, ff], ctx.dtype)
 
 

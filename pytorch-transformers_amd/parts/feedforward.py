@@ -69,8 +69,12 @@ class GatedFeedForward(Part):
     def after_load(self) -> None:
         self.inp = Linear.stacked(f"{self.name}.gate_up", [self.gate, self.up])
 
-    def forward(self, x: torch.Tensor, ctx: StepContext, add1=None, add2=None):
-        both = self.inp(x)
+    def input_projection(self):
+        """The first product of ``forward`` (see ``AttentionMixer.input_projection``)."""
+        return self.inp, {}
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, add1=None, add2=None, projected=None):
+        both = projected if projected is not None else self.inp(x)
         F = self.ffn_size
         y = ops.glu(both[:, :F], both[:, F:], self.kind, self.alpha, self.limit)
         return self.down(y, add1=as_tensor(add1), add2=as_tensor(add2))

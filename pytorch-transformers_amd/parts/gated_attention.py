@@ -85,11 +85,16 @@ class GatedAttentionMixer(Part):
         if problem is not None:
             raise ValueError(f"{self.name}: {problem}")
 
-    def forward(self, x: torch.Tensor, ctx: StepContext, call, residual: Optional[torch.Tensor] = None):
+    def input_projection(self):
+        """The first product of ``forward``: a block may run it in one launch with another part's and hand the result
+        in as ``projected``."""
+        return self.inp, {}
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, call, residual: Optional[torch.Tensor] = None, projected=None):
         k_pool, v_pool = ctx.cache.kv_layer(call.cache_group, call.cache_layer)
         table = ctx.block_tables[call.cache_group]
         H, G, dk, dv = self.num_heads, self.kv_heads, self.key_dim, self.value_dim
-        proj = self.inp(x)
+        proj = projected if projected is not None else self.inp(x)
         at = [0, H * dk, (H + G) * dk, (H + G) * dk + G * dv]
         q = ops.head_norm_rope_cache(proj[:, at[0]:at[1]], proj[:, at[1]:at[2]], proj[:, at[2]:at[3]], self.q_w, self.k_w,
                                      self.eps, self.v_norm, as_rotation(self.positions.rotation()), ctx, table, k_pool,

@@ -62,10 +62,14 @@ class DecayLinearAttentionMixer(Part):
         if self.key_dim > 256:
             raise ValueError(f"{self.name}: keys of {self.key_dim} elements are more than the 256 the kernel holds")
 
-    def forward(self, x: torch.Tensor, ctx: StepContext, call, residual: Optional[torch.Tensor] = None):
+    def input_projection(self):
+        """The first product of ``forward`` (see ``GatedAttentionMixer.input_projection``)."""
+        return self.inp, {}
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, call, residual: Optional[torch.Tensor] = None, projected=None):
         state = ctx.cache.state_layer(call.cache_group, call.cache_layer)
         H, dk, dv = self.heads, self.key_dim, self.value_dim
-        proj = self.inp(x)
+        proj = projected if projected is not None else self.inp(x)
         a, b, c = H * dk, 2 * H * dk, 2 * H * dk + H * dv
         o = ops.decay_scan(proj[:, :a], proj[:, a:b], proj[:, b:c], self.decay, state, ctx.cu_tokens, ctx.seq_slot, H, dk,
                            dv, act=self.act, max_new=max(ctx.new_tokens))

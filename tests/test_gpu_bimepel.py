@@ -384,17 +384,20 @@ def test_dense_feed_forward_clamps_its_gate(dtype, rel, rows):
 
 
 @pytest.mark.parametrize("dtype,rel", DTYPES)
-@pytest.mark.parametrize("experts,top,scale,ff", [(5, 2, 1.5, 24), (1, 1, 1.0, 8), (7, 7, 0.5, 16), (70, 3, 2.0, 40), (4, 1, 3.0, 9)])
-def test_routed_feed_forward(dtype, rel, experts, top, scale, ff):
+@pytest.mark.parametrize("experts,top,scale,ff,hidden", [(5, 2, 1.5, 24, 40), (1, 1, 1.0, 8, 40), (7, 7, 0.5, 16, 40),
+                                                         (70, 3, 2.0, 40, 40), (4, 1, 3.0, 9, 40),
+                                                         # sizes that the matrix-core launches take (steps of many tokens)
+                                                         (5, 2, 1.5, 32, 64), (70, 3, 2.0, 96, 96), (3, 3, 1.0, 160, 32)])
+def test_routed_feed_forward(dtype, rel, experts, top, scale, ff, hidden):
     from pytorch_transformers_amd import ops
     from pytorch_transformers_amd.parts import RoutedFeedForward
 
-    hidden, dt = 40, TORCH[dtype]
+    dt = TORCH[dtype]
     part = RoutedFeedForward("f", hidden, ff, experts, top, scale)
     w = _part_weights(part, seed=13, std=0.4)
     _load_part(part, w, dt)
     mlp = {"router": {"experts": experts, "top": top, "scale": scale}}
-    for rows in (1, 7, 150):
+    for rows in (1, 7, 17, 150, 700):
         x = _bf16(_rand(rows, hidden, seed=14 + rows))
         want = torch.stack([P.routed_ff(w, "f", mlp, x[i]) for i in range(rows)])
         _close(part.forward(x.to(dt).cuda(), None), want, rel, f"routed feed-forward {experts} experts top {top} rows {rows}")
