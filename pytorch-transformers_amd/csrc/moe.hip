@@ -230,109 +230,162 @@ __device__ __forceinline__ uint32_t moe_pack2(float lo, float hi) {
     return (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
 }
 
+// The products of a tile: C^T[row of W][slot] += W rows . B rows over K, for NA groups of sixteen W rows a wave and the
+// tile's four groups of sixteen slots.  W rows are the matrix cores' A operand, sixteen bytes of a row per lane,
+// straight from memory and asked for one step of 32 ahead; the tile's B rows (64 slots x 64 elements of K a stage) go
+// through LDS, which the four waves of the workgroup share, two stages in turn with one barrier a stage.
+#define MOE_STAGE 64
+#define MOE_XROW 72  // elements between two rows of a stage in LDS: 144 bytes, so that sixteen rows spread over the banks
+
+template <int NA>
+__device__ __forceinline__ void moe_tile_products(moe_f32x4_t (&acc)[NA][4], const bf16_t* const (&arow)[NA],
+                                                  const bf16_t* brow, int K, bf16_t* lds) {
+    const int tid = threadIdx.x, lane = tid & 63, c = lane & 15, gq = lane >> 4;
+    const int st_at = (tid >> 2) * MOE_XROW + (tid & 3) * 8;  // where this thread puts its two pieces of a stage
+#pragma unroll
+    for (int a = 0; a < NA; ++a)
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt) acc[a][tt] = moe_f32x4_t{0.f, 0.f, 0.f, 0.f};
+    uint4 g0 = *reinterpret_cast<const uint4*>(brow), g1 = *reinterpret_cast<const uint4*>(brow + 32);
+    MoeFrag wn[2][NA];  // the W rows' pieces of the stage to come: asked for a stage (two steps of 32) ahead
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+        for (int a = 0; a < NA; ++a) wn[ks][a].u = *reinterpret_cast<const uint4*>(arow[a] + ks * 32);
+    *reinterpret_cast<uint4*>(lds + st_at) = g0;
+    *reinterpret_cast<uint4*>(lds + st_at + 32) = g1;
+    __syncthreads();
+    const int stages = K / MOE_STAGE;
+    for (int s = 0; s < stages; ++s) {
+        const bf16_t* cur = lds + (s & 1) * (MOE_TILE * MOE_XROW);
+        const bool more = s + 1 < stages;
+        MoeFrag wc[2][NA];
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+            for (int a = 0; a < NA; ++a) wc[ks][a] = wn[ks][a];
+        if (more) {
+            g0 = *reinterpret_cast<const uint4*>(brow + (s + 1) * MOE_STAGE);
+            g1 = *reinterpret_cast<const uint4*>(brow + (s + 1) * MOE_STAGE + 32);
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+                for (int a = 0; a < NA; ++a)
+                    wn[ks][a].u = *reinterpret_cast<const uint4*>(arow[a] + (s + 1) * MOE_STAGE + ks * 32);
+        }
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            MoeFrag xb[4];
+#pragma unroll
+            for (int tt = 0; tt < 4; ++tt)
+                xb[tt].u = *reinterpret_cast<const uint4*>(cur + (tt * 16 + c) * MOE_XROW + ks * 32 + gq * 8);
+#pragma unroll
+            for (int a = 0; a < NA; ++a)
+#pragma unroll
+                for (int tt = 0; tt < 4; ++tt)
+                    acc[a][tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wc[ks][a].v, xb[tt].v, acc[a][tt], 0, 0, 0);
+        }
+        if (more) {
+            bf16_t* nxt = lds + ((s + 1) & 1) * (MOE_TILE * MOE_XROW);
+            *reinterpret_cast<uint4*>(nxt + st_at) = g0;
+            *reinterpret_cast<uint4*>(nxt + st_at + 32) = g1;
+        }
+        __syncthreads();
+    }
+}
+
+// Which (tile, block of W rows) a workgroup takes.  Workgroups go to the chip's eight dies in turn, each die with a cache
+// of its own; the tiles of one expert against one block of its rows read the same W, so they are handed to one die, one
+// after the other: workgroup L takes the L / 8-th item of die L % 8's share of the list ordered by (block, tile).
+__device__ __forceinline__ bool moe_item(int tiles, int blocks, int* tile, int* block) {
+    const int total = tiles * blocks, per = (total + 7) / 8;
+    const int L = blockIdx.x, item = (L % 8) * per + L / 8;
+    if (L / 8 >= per || item >= total) return false;
+    *block = item / tiles;
+    *tile = item - *block * tiles;
+    return true;
+}
+
+// four values of one slot's row, rows r .. r + 3 of `limit`, as bfloat16
+__device__ __forceinline__ void moe_store4(bf16_t* dst, int r, int limit, float y0, float y1, float y2, float y3) {
+    if (r + 3 < limit) {
+        uint2 w2;
+        w2.x = moe_pack2(y0, y1);
+        w2.y = moe_pack2(y2, y3);
+        *reinterpret_cast<uint2*>(dst) = w2;
+    } else {
+        const float y[4] = {y0, y1, y2, y3};
+        for (int j = 0; j < 4; ++j)
+            if (r + j < limit) dst[j] = f32_to_bf16_bits(y[j]);
+    }
+}
+
 // act_sorted[slot, f] = act(G_e x) * (U_e x) for the slot's pair (token, e).  A workgroup of four waves owns a tile of
-// MOE_TILE slots and 64 rows f of its expert; a wave owns sixteen rows of the gate and the same sixteen of the up
-// matrix against all four groups of sixteen tokens: W rows are the A operand (sixteen bytes of a row per lane), x rows
-// the B operand, both straight from memory (the four waves read the same x rows, which the caches hold).
+// MOE_TILE slots and 128 rows f of its expert; a wave 32 rows of the gate and the same 32 of the up matrix.
 __global__ __launch_bounds__(256) void moe_grouped_up_kernel(bf16_t* __restrict__ act_sorted, const bf16_t* __restrict__ x,
                                                              long x_ld, const bf16_t* __restrict__ gate_up,
                                                              const int* __restrict__ sorted_pair,
                                                              const int* __restrict__ tile_expert, int H, int F, int top,
-                                                             int act) {
-    const int tile = blockIdx.x, e = tile_expert[tile];
+                                                             int act, int tiles) {
+    __shared__ __attribute__((aligned(16))) bf16_t lds[2 * MOE_TILE * MOE_XROW];
+    int tile, fb;
+    if (!moe_item(tiles, (F + 127) / 128, &tile, &fb)) return;
+    const int e = tile_expert[tile];
     if (e < 0) return;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, gq = lane >> 4;
-    const int f0 = blockIdx.y * 64 + wave * 16;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, c = lane & 15, gq = lane >> 4;
+    const int f0 = fb * 128 + wave * 32;
+    const bf16_t* W = gate_up + (long)e * 2 * F * H + gq * 8;
+    const bf16_t* arow[4];
+#pragma unroll
+    for (int a = 0; a < 4; ++a)  // gate rows f0 .. f0 + 31, then the same rows of the up matrix
+        arow[a] = W + ((long)(a >> 1) * F + min(f0 + (a & 1) * 16 + c, F - 1)) * H;
+    const int pair = sorted_pair[tile * MOE_TILE + (tid >> 2)];
+    const bf16_t* brow = x + (long)(pair < 0 ? 0 : pair / top) * x_ld + (tid & 3) * 8;
+    moe_f32x4_t acc[4][4];
+    moe_tile_products<4>(acc, arow, brow, H, lds);
     if (f0 >= F) return;
-    const int fr = min(f0 + c, F - 1);
-    const bf16_t* G = gate_up + ((long)e * 2 * F + fr) * H + gq * 8;
-    const bf16_t* U = G + (long)F * H;
-    const bf16_t* xr[4];
-#pragma unroll
-    for (int tt = 0; tt < 4; ++tt) {
-        const int pair = sorted_pair[tile * MOE_TILE + tt * 16 + c];
-        xr[tt] = x + (long)(pair < 0 ? 0 : pair / top) * x_ld + gq * 8;
-    }
-    moe_f32x4_t ag[4], au[4];
-#pragma unroll
-    for (int tt = 0; tt < 4; ++tt) { ag[tt] = moe_f32x4_t{0.f, 0.f, 0.f, 0.f}; au[tt] = moe_f32x4_t{0.f, 0.f, 0.f, 0.f}; }
-    for (int k = 0; k < H; k += 32) {
-        MoeFrag wg, wu, xb[4];
-        wg.u = *reinterpret_cast<const uint4*>(G + k);
-        wu.u = *reinterpret_cast<const uint4*>(U + k);
-#pragma unroll
-        for (int tt = 0; tt < 4; ++tt) xb[tt].u = *reinterpret_cast<const uint4*>(xr[tt] + k);
-#pragma unroll
-        for (int tt = 0; tt < 4; ++tt) {
-            ag[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wg.v, xb[tt].v, ag[tt], 0, 0, 0);
-            au[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wu.v, xb[tt].v, au[tt], 0, 0, 0);
-        }
-    }
-    // acc[j] is row f0 + 4 gq + j of the token in column c
-#pragma unroll
-    for (int tt = 0; tt < 4; ++tt) {
-        const long slot = (long)tile * MOE_TILE + tt * 16 + c;
-        float y[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) y[j] = apply_act(round_to_bf16(ag[tt][j]), act) * round_to_bf16(au[tt][j]);
-        bf16_t* dst = act_sorted + slot * F + f0 + 4 * gq;
-        if (f0 + 4 * gq + 3 < F) {
-            uint2 w2;
-            w2.x = moe_pack2(y[0], y[1]);
-            w2.y = moe_pack2(y[2], y[3]);
-            *reinterpret_cast<uint2*>(dst) = w2;
-        } else {
-            for (int j = 0; j < 4; ++j)
-                if (f0 + 4 * gq + j < F) dst[j] = f32_to_bf16_bits(y[j]);
-        }
-    }
-}
-
-// y_sorted[slot, n] = D_e act_sorted[slot]: a wave owns two groups of sixteen rows n of the expert's down matrix against
-// the tile's four groups of sixteen slots; a workgroup 128 rows
-__global__ __launch_bounds__(256) void moe_grouped_down_kernel(bf16_t* __restrict__ y_sorted, const bf16_t* __restrict__ act_sorted,
-                                                               const bf16_t* __restrict__ down,
-                                                               const int* __restrict__ tile_expert, int H, int F) {
-    const int tile = blockIdx.x, e = tile_expert[tile];
-    if (e < 0) return;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, gq = lane >> 4;
-    const int n0 = blockIdx.y * 128 + wave * 32;
-    if (n0 >= H) return;
-    const bf16_t* D0 = down + ((long)e * H + min(n0 + c, H - 1)) * F + gq * 8;
-    const bf16_t* D1 = down + ((long)e * H + min(n0 + 16 + c, H - 1)) * F + gq * 8;
-    const bf16_t* ar = act_sorted + ((long)tile * MOE_TILE + c) * F + gq * 8;
-    moe_f32x4_t a0[4], a1[4];
-#pragma unroll
-    for (int tt = 0; tt < 4; ++tt) { a0[tt] = moe_f32x4_t{0.f, 0.f, 0.f, 0.f}; a1[tt] = moe_f32x4_t{0.f, 0.f, 0.f, 0.f}; }
-    for (int k = 0; k < F; k += 32) {
-        MoeFrag w0, w1, xb[4];
-        w0.u = *reinterpret_cast<const uint4*>(D0 + k);
-        w1.u = *reinterpret_cast<const uint4*>(D1 + k);
-#pragma unroll
-        for (int tt = 0; tt < 4; ++tt) xb[tt].u = *reinterpret_cast<const uint4*>(ar + (long)tt * 16 * F + k);
-#pragma unroll
-        for (int tt = 0; tt < 4; ++tt) {
-            a0[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0.v, xb[tt].v, a0[tt], 0, 0, 0);
-            a1[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1.v, xb[tt].v, a1[tt], 0, 0, 0);
-        }
-    }
+    // acc[a][tt][j] is row f0 + (a & 1) * 16 + 4 gq + j of the slot in column c of group tt
 #pragma unroll
     for (int tt = 0; tt < 4; ++tt) {
         const long slot = (long)tile * MOE_TILE + tt * 16 + c;
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
-            const moe_f32x4_t& a = half ? a1[tt] : a0[tt];
-            const int n = n0 + half * 16 + 4 * gq;
-            bf16_t* dst = y_sorted + slot * H + n;
-            if (n + 3 < H) {
-                uint2 w2;
-                w2.x = moe_pack2(a[0], a[1]);
-                w2.y = moe_pack2(a[2], a[3]);
-                *reinterpret_cast<uint2*>(dst) = w2;
-            } else {
-                for (int j = 0; j < 4; ++j)
-                    if (n + j < H) dst[j] = f32_to_bf16_bits(a[j]);
-            }
+            float y[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                y[j] = apply_act(round_to_bf16(acc[half][tt][j]), act) * round_to_bf16(acc[2 + half][tt][j]);
+            const int f = f0 + half * 16 + 4 * gq;
+            moe_store4(act_sorted + slot * F + f, f, F, y[0], y[1], y[2], y[3]);
+        }
+    }
+}
+
+// y_sorted[slot, n] = D_e act_sorted[slot]: a wave owns four groups of sixteen rows n of the expert's down matrix, a
+// workgroup 256 rows, against the tile's 64 slots
+__global__ __launch_bounds__(256) void moe_grouped_down_kernel(bf16_t* __restrict__ y_sorted, const bf16_t* __restrict__ act_sorted,
+                                                               const bf16_t* __restrict__ down,
+                                                               const int* __restrict__ tile_expert, int H, int F, int tiles) {
+    __shared__ __attribute__((aligned(16))) bf16_t lds[2 * MOE_TILE * MOE_XROW];
+    int tile, nb;
+    if (!moe_item(tiles, (H + 255) / 256, &tile, &nb)) return;
+    const int e = tile_expert[tile];
+    if (e < 0) return;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, c = lane & 15, gq = lane >> 4;
+    const int n0 = nb * 256 + wave * 64;
+    const bf16_t* arow[4];
+#pragma unroll
+    for (int a = 0; a < 4; ++a) arow[a] = down + ((long)e * H + min(n0 + a * 16 + c, H - 1)) * F + gq * 8;
+    const bf16_t* brow = act_sorted + ((long)tile * MOE_TILE + (tid >> 2)) * F + (tid & 3) * 8;
+    moe_f32x4_t acc[4][4];
+    moe_tile_products<4>(acc, arow, brow, F, lds);
+    if (n0 >= H) return;
+#pragma unroll
+    for (int tt = 0; tt < 4; ++tt) {
+        const long slot = (long)tile * MOE_TILE + tt * 16 + c;
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+            const int n = n0 + a * 16 + 4 * gq;
+            moe_store4(y_sorted + slot * H + n, n, H, acc[a][tt][0], acc[a][tt][1], acc[a][tt][2], acc[a][tt][3]);
         }
     }
 }
@@ -351,13 +404,13 @@ __global__ void moe_combine_kernel(bf16_t* __restrict__ out, const bf16_t* __res
 
 extern "C" int pta_moe_grouped_slots(int pairs, int E) { return (pairs + E * (MOE_TILE - 1) + MOE_TILE - 1) / MOE_TILE * MOE_TILE; }
 
-// bfloat16 only; H and F multiples of 32.  sorted_pair [slots], slot_of_pair [M * top], tile_expert [slots / 64],
+// bfloat16 only; H and F multiples of 64.  sorted_pair [slots], slot_of_pair [M * top], tile_expert [slots / 64],
 // act_sorted [slots, F], y_sorted [slots, H] are the caller's scratch (slots = pta_moe_grouped_slots(M * top, E)).
 extern "C" int pta_moe_grouped(void* out, const void* x, long x_ld, const void* gate_up, const void* down, const int* ids,
                                const float* wts, int* sorted_pair, int* slot_of_pair, int* tile_expert, void* act_sorted,
                                void* y_sorted, int M, int H, int F, int E, int top, int act, void* stream) {
     PTA_REQUIRE(M > 0 && H > 0 && F > 0 && E > 0 && top > 0, "moe_grouped: sizes must be positive");
-    PTA_REQUIRE(H % 32 == 0 && F % 32 == 0 && x_ld % 8 == 0, "moe_grouped: features (%d) and expert size (%d) must be multiples of 32", H, F);
+    PTA_REQUIRE(H % 64 == 0 && F % 64 == 0 && x_ld % 8 == 0, "moe_grouped: features (%d) and expert size (%d) must be multiples of 64", H, F);
     PTA_REQUIRE(out && x && gate_up && down && ids && wts && sorted_pair && slot_of_pair && tile_expert && act_sorted && y_sorted,
                 "moe_grouped: null pointer");
     PTA_REQUIRE((((uintptr_t)x | (uintptr_t)gate_up | (uintptr_t)down | (uintptr_t)act_sorted | (uintptr_t)y_sorted) % 16) == 0,
@@ -370,10 +423,11 @@ extern "C" int pta_moe_grouped(void* out, const void* x, long x_ld, const void* 
     hipStream_t s = (hipStream_t)stream;
     hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), (size_t)(3 * E + 1) * 4, s, sorted_pair, slot_of_pair, tile_expert,
                        ids, (int)pairs, E, slots, tiles);
-    hipLaunchKernelGGL(moe_grouped_up_kernel, dim3(tiles, (F + 63) / 64), dim3(256), 0, s, (bf16_t*)act_sorted, (const bf16_t*)x,
-                       x_ld, (const bf16_t*)gate_up, sorted_pair, tile_expert, H, F, top, act);
-    hipLaunchKernelGGL(moe_grouped_down_kernel, dim3(tiles, (H + 127) / 128), dim3(256), 0, s, (bf16_t*)y_sorted,
-                       (const bf16_t*)act_sorted, (const bf16_t*)down, tile_expert, H, F);
+    auto grid_for = [&](int blocks) { return dim3((unsigned)(((long)tiles * blocks + 7) / 8 * 8)); };
+    hipLaunchKernelGGL(moe_grouped_up_kernel, grid_for((F + 127) / 128), dim3(256), 0, s, (bf16_t*)act_sorted, (const bf16_t*)x,
+                       x_ld, (const bf16_t*)gate_up, sorted_pair, tile_expert, H, F, top, act, tiles);
+    hipLaunchKernelGGL(moe_grouped_down_kernel, grid_for((H + 255) / 256), dim3(256), 0, s, (bf16_t*)y_sorted,
+                       (const bf16_t*)act_sorted, (const bf16_t*)down, tile_expert, H, F, tiles);
     hipLaunchKernelGGL(moe_combine_kernel, dim3(M), dim3(256), 0, s, (bf16_t*)out, (const bf16_t*)y_sorted, slot_of_pair, wts, H, top);
     return pta_check_launch("moe_grouped");
 }

@@ -1593,7 +1593,7 @@ def moe_experts(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, ids:
     ld = _rows_of(h, "h", H, h.dtype)
     out = torch.empty((M, H), dtype=h.dtype, device=h.device)
     timing_hint["experts"] = E
-    if (h.dtype == torch.bfloat16 and M > MOE_GROUPED_FROM_ROWS and H % 32 == 0 and F % 32 == 0 and ld % 8 == 0
+    if (h.dtype == torch.bfloat16 and M > MOE_GROUPED_FROM_ROWS and H % 64 == 0 and F % 64 == 0 and ld % 8 == 0
             and h.data_ptr() % 16 == 0):
         # many tokens: the pairs sorted by expert, tiles of one expert's tokens on the matrix cores
         slots = load_library().pta_moe_grouped_slots(M * top, E)

@@ -387,7 +387,7 @@ def test_dense_feed_forward_clamps_its_gate(dtype, rel, rows):
 @pytest.mark.parametrize("experts,top,scale,ff,hidden", [(5, 2, 1.5, 24, 40), (1, 1, 1.0, 8, 40), (7, 7, 0.5, 16, 40),
                                                          (70, 3, 2.0, 40, 40), (4, 1, 3.0, 9, 40),
                                                          # sizes that the matrix-core launches take (steps of many tokens)
-                                                         (5, 2, 1.5, 32, 64), (70, 3, 2.0, 96, 96), (3, 3, 1.0, 160, 32)])
+                                                         (5, 2, 1.5, 64, 64), (70, 3, 2.0, 192, 128), (3, 3, 1.0, 320, 64)])
 def test_routed_feed_forward(dtype, rel, experts, top, scale, ff, hidden):
     from pytorch_transformers_amd import ops
     from pytorch_transformers_amd.parts import RoutedFeedForward
