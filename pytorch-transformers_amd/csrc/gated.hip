@@ -10,8 +10,10 @@
 #include "common.h"
 #include "pta_kernels.h"
 
+#include <algorithm>
+
 template <typename T, typename TX>
-__global__ __launch_bounds__(256) void gated_heads_kernel(T* __restrict__ out, const TX* __restrict__ x, long x_ld,
+__global__ __launch_bounds__(1024) void gated_heads_kernel(T* __restrict__ out, const TX* __restrict__ x, long x_ld,
                                                           int x_head, const T* __restrict__ g, long g_ld,
                                                           const float* __restrict__ w, float eps, int heads, int dv) {
     __shared__ float red[16];
@@ -43,7 +45,7 @@ extern "C" int pta_gated_heads(void* out, const void* x, int x_f32, long x_ld, i
                 "gated_heads: rows or frames lie closer together than they are long");
     PTA_REQUIRE(dtype == PTA_F32 || dtype == PTA_BF16, "gated_heads: unknown dtype %d", dtype);
     hipStream_t s = (hipStream_t)stream;
-    const dim3 grid(M), block(heads * dv >= 1024 ? 256 : 64);
+    const dim3 grid(M), block(std::min(1024, std::max(64, (heads * dv / 4 + 63) / 64 * 64)));
     if (dtype == PTA_F32)
         hipLaunchKernelGGL((gated_heads_kernel<float, float>), grid, block, 0, s, (float*)out, (const float*)x, x_ld, x_head,
                            (const float*)g, g_ld, w, eps, heads, dv);

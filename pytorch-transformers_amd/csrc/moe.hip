@@ -42,7 +42,7 @@ __device__ __forceinline__ float wave_dot(const T* __restrict__ w, const float* 
 }
 
 template <typename T>
-__global__ __launch_bounds__(256) void moe_route_kernel(int* __restrict__ ids, float* __restrict__ wts,
+__global__ __launch_bounds__(1024) void moe_route_kernel(int* __restrict__ ids, float* __restrict__ wts,
                                                         const T* __restrict__ h, long h_ld, const float* __restrict__ Wr,
                                                         int H, int E, int top, int score_kind, int normalise, float scale) {
     extern __shared__ __attribute__((aligned(16))) float sm[];
@@ -105,10 +105,11 @@ extern "C" int pta_moe_route(int* ids, float* wts, const void* h, long h_ld, con
     PTA_REQUIRE(dtype == PTA_F32 || dtype == PTA_BF16, "moe_route: unknown dtype %d", dtype);
     hipStream_t s = (hipStream_t)stream;
     const size_t lds = (size_t)(H + E) * sizeof(float);
+    const dim3 block(E >= 16 ? 1024 : E >= 8 ? 512 : 256);  // a wave an expert where there are that many
     if (dtype == PTA_F32)
-        hipLaunchKernelGGL(moe_route_kernel<float>, dim3(M), dim3(256), lds, s, ids, wts, (const float*)h, h_ld, Wr, H, E, top, score_kind, normalise, scale);
+        hipLaunchKernelGGL(moe_route_kernel<float>, dim3(M), block, lds, s, ids, wts, (const float*)h, h_ld, Wr, H, E, top, score_kind, normalise, scale);
     else
-        hipLaunchKernelGGL(moe_route_kernel<bf16_t>, dim3(M), dim3(256), lds, s, ids, wts, (const bf16_t*)h, h_ld, Wr, H, E, top, score_kind, normalise, scale);
+        hipLaunchKernelGGL(moe_route_kernel<bf16_t>, dim3(M), block, lds, s, ids, wts, (const bf16_t*)h, h_ld, Wr, H, E, top, score_kind, normalise, scale);
     return pta_check_launch("moe_route");
 }
 

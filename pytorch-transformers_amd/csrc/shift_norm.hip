@@ -13,6 +13,8 @@
 #include "common.h"
 #include "pta_kernels.h"
 
+#include <algorithm>
+
 enum { PTA_SHIFT_TOKENS = 0, PTA_SHIFT_STATE = 1 };
 
 template <typename T>
@@ -27,7 +29,7 @@ __device__ __forceinline__ float row_value(const float* base, const T* t1, const
 }
 
 template <typename T>
-__global__ __launch_bounds__(256) void shift_norm_kernel(
+__global__ __launch_bounds__(1024) void shift_norm_kernel(
     T* __restrict__ a_out, T* __restrict__ m_out, float* __restrict__ x_out, const float* __restrict__ base,
     const T* __restrict__ t1, const T* __restrict__ t2, const float* __restrict__ w1, const float* __restrict__ w2,
     const float* __restrict__ mu, float* __restrict__ state, long state_ld, const int* __restrict__ token_seq,
@@ -98,7 +100,8 @@ extern "C" int pta_shift_norm(void* a_out, void* m_out, float* x_out, const floa
     PTA_REQUIRE(H <= 16384, "shift_norm: rows of %d features are more than the 16384 that fit the kernel's LDS", H);
     PTA_REQUIRE(dtype == PTA_F32 || dtype == PTA_BF16, "shift_norm: unknown dtype %d", dtype);
     hipStream_t s = (hipStream_t)stream;
-    const dim3 block(H >= 1024 ? 256 : H >= 256 ? 128 : 64);
+    // a thread takes four features or so: a row's loads are then few rounds of many, not many rounds of few
+    const dim3 block(std::min(1024, std::max(64, (H / 4 + 63) / 64 * 64)));
     const size_t lds = (size_t)2 * H * sizeof(float);
     if (lds > 64 * 1024) {
         if (dtype == PTA_F32)
