@@ -118,15 +118,29 @@ __global__ void la_carry_kernel(float* __restrict__ state, long state_ld, float*
     const float a = decay[h];
     float* sp = state + (long)seq_slot[s] * state_ld + e;
     float S = *sp;
-    for (int c = 0; c < n_chunks; ++c) {
-        const long seg = (long)s * max_chunks + c;
-        float* cs = chunk_state + seg * heads * hs + e;
-        const float add = *cs;
-        *cs = S;
-        const int len = min(chunk, n_new - c * chunk);
-        float pw = 1.f;  // decay^len as the chunk's own walk multiplies it up
-        for (int i = 0; i < len; ++i) pw *= a;
-        S = pw * S + add;
+    const long step = (long)heads * hs;  // from a chunk's element to the next chunk's
+    float* cs = chunk_state + (long)s * max_chunks * step + e;
+    float pw_full = 1.f;  // decay^chunk as the chunks' own walks multiply it up
+    for (int i = 0; i < chunk; ++i) pw_full *= a;
+    // eight chunks' additions are asked for at once: the walk itself is a chain, its loads need not be
+    for (int c0 = 0; c0 < n_chunks; c0 += 8) {
+        float add[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) add[j] = c0 + j < n_chunks ? cs[(long)(c0 + j) * step] : 0.f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int c = c0 + j;
+            if (c < n_chunks) {
+                cs[(long)c * step] = S;
+                float pw = pw_full;
+                const int len = n_new - c * chunk;
+                if (len < chunk) {
+                    pw = 1.f;
+                    for (int i = 0; i < len; ++i) pw *= a;
+                }
+                S = pw * S + add[j];
+            }
+        }
     }
     *sp = S;
 }
