@@ -41,6 +41,40 @@ __device__ __forceinline__ float wave_dot(const T* __restrict__ w, const float* 
     return wave_sum(acc);
 }
 
+// the same for NR rows of W `row_ld` apart at once, so that NR loads are on their way for every step over K
+template <typename T, int NR>
+__device__ __forceinline__ void wave_dots(const T* __restrict__ w, long row_ld, int rows, const float* __restrict__ x_s, int K,
+                                          int lane, float (&out)[NR]) {
+    float acc[NR];
+#pragma unroll
+    for (int r = 0; r < NR; ++r) acc[r] = 0.f;
+    const T* wr[NR];
+#pragma unroll
+    for (int r = 0; r < NR; ++r) wr[r] = w + (long)min(r, rows - 1) * row_ld;  // rows past the last repeat it
+    if (sizeof(T) == 2 && (K & 7) == 0 && ((uintptr_t)w & 15) == 0 && (row_ld & 7) == 0) {
+#pragma unroll 2
+        for (int k = lane * 8; k < K; k += PTA_WAVE * 8) {
+            uint4 u[NR];
+#pragma unroll
+            for (int r = 0; r < NR; ++r) u[r] = *reinterpret_cast<const uint4*>((const bf16_t*)wr[r] + k);
+            const float4 x0 = *reinterpret_cast<const float4*>(x_s + k), x1 = *reinterpret_cast<const float4*>(x_s + k + 4);
+#pragma unroll
+            for (int r = 0; r < NR; ++r) {
+                float f[8];
+                unpack8(u[r], f);
+                acc[r] += f[0] * x0.x + f[1] * x0.y + f[2] * x0.z + f[3] * x0.w + f[4] * x1.x + f[5] * x1.y + f[6] * x1.z + f[7] * x1.w;
+            }
+        }
+    } else {
+        for (int k = lane; k < K; k += PTA_WAVE) {
+#pragma unroll
+            for (int r = 0; r < NR; ++r) acc[r] += Io<T>::ld(wr[r] + k) * x_s[k];
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < NR; ++r) out[r] = wave_sum(acc[r]);
+}
+
 template <typename T>
 __global__ __launch_bounds__(1024) void moe_route_kernel(int* __restrict__ ids, float* __restrict__ wts,
                                                         const T* __restrict__ h, long h_ld, const float* __restrict__ Wr,
@@ -126,11 +160,19 @@ __global__ __launch_bounds__(256) void moe_up_kernel(T* __restrict__ act_out, co
     __syncthreads();
     const T* G = gate_up + (long)e * 2 * F * H;
     const T* U = G + (long)F * H;
-    for (int f = blockIdx.y * MOE_ROWS + wave; f < min(F, (int)(blockIdx.y + 1) * MOE_ROWS); f += 4) {
-        const float g = wave_dot<T>(G + (long)f * H, x_s, H, lane);
-        const float u = wave_dot<T>(U + (long)f * H, x_s, H, lane);
-        // (each product rounded to the compute type first, as a product on its own would leave it)
-        if (lane == 0) Io<T>::st(act_out + (long)pair * F + f, apply_act(Io<T>::round(g), act) * Io<T>::round(u));
+    // a wave takes four neighbouring rows of the gate and of the up matrix: eight loads on their way at once
+    const int f0 = blockIdx.y * MOE_ROWS + wave * 4, rows = min(4, F - f0);
+    if (rows <= 0) return;
+    float g[4], u[4];
+    wave_dots<T, 4>(G + (long)f0 * H, H, rows, x_s, H, lane, g);
+    wave_dots<T, 4>(U + (long)f0 * H, H, rows, x_s, H, lane, u);
+    // (each product rounded to the compute type first, as a product on its own would leave it)
+    if (lane < rows) {
+        float gv = g[0], uv = u[0];
+#pragma unroll
+        for (int r = 1; r < 4; ++r)
+            if (lane == r) { gv = g[r]; uv = u[r]; }
+        Io<T>::st(act_out + (long)pair * F + f0 + lane, apply_act(Io<T>::round(gv), act) * Io<T>::round(uv));
     }
 }
 
@@ -142,13 +184,22 @@ __global__ __launch_bounds__(256) void moe_down_kernel(T* __restrict__ out, cons
     const int m = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     for (int i = threadIdx.x; i < top * F; i += blockDim.x) a_s[i] = Io<T>::ld(act_in + (long)m * top * F + i);
     __syncthreads();
-    for (int n = blockIdx.y * MOE_ROWS + wave; n < min(H, (int)(blockIdx.y + 1) * MOE_ROWS); n += 4) {
-        float acc = 0.f;
-        for (int k = 0; k < top; ++k) {
-            const T* D = down + ((long)ids[(long)m * top + k] * H + n) * F;
-            acc += wts[(long)m * top + k] * Io<T>::round(wave_dot<T>(D, a_s + k * F, F, lane));
-        }
-        if (lane == 0) Io<T>::st(out + (long)m * H + n, acc);
+    const int n0 = blockIdx.y * MOE_ROWS + wave * 4, rows = min(4, H - n0);
+    if (rows <= 0) return;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int k = 0; k < top; ++k) {
+        float d[4];
+        wave_dots<T, 4>(down + ((long)ids[(long)m * top + k] * H + n0) * F, F, rows, a_s + k * F, F, lane, d);
+        const float wk = wts[(long)m * top + k];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[r] += wk * Io<T>::round(d[r]);
+    }
+    if (lane < rows) {
+        float v = acc[0];
+#pragma unroll
+        for (int r = 1; r < 4; ++r)
+            if (lane == r) v = acc[r];
+        Io<T>::st(out + (long)m * H + n0 + lane, v);
     }
 }
 
