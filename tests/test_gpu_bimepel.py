@@ -566,3 +566,78 @@ def test_the_command_line_generates_from_a_model_folder(tmp_path, capsys):
     for _ in range(6):
         toks.append(int(P.PlainBimepel(cfg, w).logits(toks)[-1].argmax()))
     assert [int(t) for t in printed[-1].split(",")] == toks
+
+
+# ---- configurations drawn at random ------------------------------------------------------------------------------------
+def draw_config(seed):
+    """A small model with sizes that nothing else here hits: widths and feed-forwards that are no multiple of 8, head
+    sizes from 8 to 130, head counts and groups that are no power of two, rotations of two elements up to the whole
+    head, with and without the ramp, masks of any size, decays up to one, one to nine experts, loops anywhere."""
+    import random
+
+    r = random.Random(seed)
+    width = r.choice([20, 36, 44, 48, 64, 72, 100])
+
+    def layer():
+        if r.random() < 0.55:
+            kv = r.choice([1, 2, 3])
+            dim = r.choice([8, 12, 16, 24, 40, 64, 72, 130])
+            m = {"heads": kv * r.choice([1, 2, 3, 5]), "kv_heads": kv, "dim": dim,
+                 "vdim": r.choice([4, 8, 20, 32, 48, 64, 100]), "scale": r.choice([0.1, 0.25, dim ** -0.5])}
+            if r.random() < 0.85:
+                m["rot"] = {"base": r.choice([100.0, 1e4, 250000.0]), "dims": r.choice([2, dim // 2 // 2 * 2 or 2, dim])}
+                if r.random() < 0.6:
+                    m["rot"]["scaling"] = {"factor": r.choice([2.0, 8.0]), "original": r.choice([16, 64, 2048]),
+                                           "fast": r.choice([32.0, 4.0]), "slow": r.choice([1.0, 0.5])}
+            if r.random() < 0.8:
+                m["mask"] = {"size": r.choice([1, 3, 16, 33, 64, 65, 128, 1000])}
+            out = {"type": "attention", "mixer": m}
+        else:
+            heads = r.choice([1, 2, 3, 5])
+            out = {"type": "lightning", "mixer": {"heads": heads, "dim": r.choice([4, 8, 20, 32, 70]),
+                                                  "vdim": r.choice([4, 16, 24, 64, 80]),
+                                                  "decay": [r.choice([0.3, 0.9, 0.99, 0.999, 1.0]) for _ in range(heads)]}}
+        kind = r.random()
+        if kind < 0.15:
+            out["mlp"] = None
+        elif kind < 0.55:
+            out["mlp"] = {"kind": "dense", "ff": r.choice([8, 20, 50, 96]), "limit": r.choice([0.5, 1.0, 7.0])}
+        else:
+            experts = r.choice([1, 2, 4, 9])
+            out["mlp"] = {"kind": "moe", "expert": {"ff": r.choice([4, 12, 32, 64])},
+                          "router": {"experts": experts, "top": r.randint(1, experts), "scale": r.choice([0.5, 1.0, 2.5])}}
+        return out
+
+    n = r.choice([1, 2, 3, 4])
+    cfg = config([layer() for _ in range(n)], vocab=r.choice([61, 97, 211]), width=width, eps=r.choice([1e-5, 1e-6]))
+    if r.random() < 0.7:
+        a = r.randint(0, n - 1)
+        cfg["loop"] = {"start": a, "stop": r.randint(a, n), "times": r.choice([1, 2, 3])}
+    return cfg
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_configurations_drawn_at_random(tmp_path, seed):
+    """Whole, cut and batched against the plain model in 32-bit; bfloat16 runs and agrees with itself across schedules
+    to rounding (it is held against the plain model where the sizes are the tests' own, above)."""
+    from pytorch_transformers_amd.engine.replay import Replayer
+
+    cfg = draw_config(seed)
+    w = make_weights(cfg, seed=100 + seed)
+    folder = write_model(tmp_path / "m", cfg, w)
+    reqs = helpers.make_requests(cfg["vocab"], [5, 70, 140, 1, 66], seed=seed)
+    want = plain_all(cfg, w, reqs)
+    model = load(folder, "float32")
+    rp = Replayer(model, 1024, max_slots=8)
+    for label, records in (("whole", helpers.schedule_whole(reqs)), ("batches", helpers.schedule_batches(reqs, 3)),
+                           ("staggered", helpers.schedule_staggered(reqs, chunks=(None, 2, 19, 1)))):
+        got = helpers.run_schedule(rp, records)
+        for rid in reqs:
+            helpers.assert_close(got[rid], want[rid], helpers.REL_F32, f"seed {seed} {label} {rid}: {cfg}")
+    model = load(folder, "bfloat16")
+    rp = Replayer(model, 1024, max_slots=8)
+    whole = helpers.run_schedule(rp, helpers.schedule_whole(reqs))
+    cut = helpers.run_schedule(rp, helpers.schedule_staggered(reqs, chunks=(None, 2, 19, 1)))
+    for rid in reqs:
+        assert torch.isfinite(whole[rid]).all()
+        assert_model_close(cut[rid], whole[rid], 0.15, f"seed {seed} bfloat16, cut against whole, {rid}: {cfg}")
