@@ -223,9 +223,15 @@ extern "C" int pta_moe_up(void* act_out, const void* h, long h_ld, const void* g
 extern "C" int pta_moe_down(void* out, const void* act_in, const void* down, const int* ids, const float* wts, int M, int H,
                             int F, int top, int dtype, void* stream) {
     PTA_REQUIRE(M > 0 && H > 0 && F > 0 && top > 0 && out && act_in && down && ids && wts, "moe_down: sizes must be positive and pointers given");
-    PTA_REQUIRE((size_t)top * F * 4 <= 64 * 1024 && (H + MOE_ROWS - 1) / MOE_ROWS <= 65535, "moe_down: sizes beyond one launch");
+    PTA_REQUIRE((size_t)top * F * 4 <= 160 * 1024 && (H + MOE_ROWS - 1) / MOE_ROWS <= 65535,
+                "moe_down: %d experts of %d rows a token are more than the kernel's LDS holds", top, F);
     PTA_REQUIRE(dtype == PTA_F32 || dtype == PTA_BF16, "moe_down: unknown dtype %d", dtype);
     hipStream_t s = (hipStream_t)stream;
+    if ((size_t)top * F * 4 > 64 * 1024) {  // more than a launch may ask for unless the kernel has been told
+        const void* kern = dtype == PTA_F32 ? reinterpret_cast<const void*>(moe_down_kernel<float>)
+                                            : reinterpret_cast<const void*>(moe_down_kernel<bf16_t>);
+        (void)hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)((size_t)top * F * 4));
+    }
     const dim3 grid(M, (H + MOE_ROWS - 1) / MOE_ROWS);
     if (dtype == PTA_F32)
         hipLaunchKernelGGL(moe_down_kernel<float>, grid, dim3(256), (size_t)top * F * 4, s, (float*)out, (const float*)act_in, (const float*)down, ids, wts, H, F, top);
