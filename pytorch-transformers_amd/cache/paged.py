@@ -20,7 +20,9 @@ state table one more row (``scratch_page``, ``scratch_slot``) that no sequence e
 step to a fixed batch size (a captured decode step) write there, so that padding touches no sequence's
 keys, values or state.  A group of kind ``window`` is laid out like a full one, but gives the pages that lie
 wholly behind its window back to its pool as a sequence grows (their places in the page list hold
--1), so a long sequence holds about ``window / page_size`` pages of it.  Groups of kind ``state`` own a ``[max_slots, *shape]`` table per
+-1), so a long sequence holds about ``window / page_size`` pages of it.  A group of kind ``chunk`` (tokens see the keys of
+their own block of ``chunk`` positions only) does the same with the pages that lie wholly before the block of the
+sequence's next token.  Groups of kind ``state`` own a ``[max_slots, *shape]`` table per
 layer that is zeroed when a slot is handed out.
 
 The K pool has the layout ``[layer, page, kv_head, page_size, head_dim]``, the V pool
@@ -35,7 +37,7 @@ from typing import Dict, List, Optional, Sequence
 import torch
 
 from .. import host
-from ..engine.spec import CACHE_FULL, CACHE_STATE, CACHE_WINDOW, CacheGroupSpec
+from ..engine.spec import CACHE_CHUNK, CACHE_FULL, CACHE_STATE, CACHE_WINDOW, CacheGroupSpec
 
 PAGE_SIZE = 64
 
@@ -56,8 +58,11 @@ class _Group:
         self.page_size = page_size
         self.k = self.v = None
         self.state: Optional[torch.Tensor] = None
-        self.paged = spec.kind in (CACHE_FULL, CACHE_WINDOW)
+        self.paged = spec.kind in (CACHE_FULL, CACHE_WINDOW, CACHE_CHUNK)
         self.window = int(spec.window or 0) if spec.kind == CACHE_WINDOW else 0
+        self.chunk = int(spec.chunk or 0) if spec.kind == CACHE_CHUNK else 0
+        if spec.kind == CACHE_CHUNK and self.chunk <= 0:
+            raise CacheError(f"cache group {spec.name!r}: kind 'chunk' needs a positive block size, got {spec.chunk!r}")
         self.index = -1  # among the paged groups, as the host runtime counts them
         if spec.kind == CACHE_WINDOW and self.window <= 0:
             raise CacheError(f"cache group {spec.name!r}: kind 'window' needs a positive window, got {spec.window!r}")
@@ -102,6 +107,10 @@ class PagedCache:
                                            host.int_array([self.groups[n].window for n in self._paged]))
         if not self._h:
             raise CacheError(host.last_error())
+        for name in self._paged:
+            g = self.groups[name]
+            if g.chunk and self._lib.ptah_cache_set_chunk(self._h, g.index, g.chunk):
+                raise CacheError(host.last_error())
 
     def __del__(self):
         h, self._h = getattr(self, "_h", None), None

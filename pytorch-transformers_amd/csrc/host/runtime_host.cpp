@@ -69,6 +69,7 @@ struct Group {
     FreeList pages;
     std::vector<std::vector<int>> lists;  // per slot: page of every 64 positions, -1 where a window has moved on
     int window = 0;                        // 0: all keys are kept; w: a token sees the last w positions only
+    int chunk = 0;                         // 0, or c: a token sees the keys of its own block of c positions only
 };
 
 struct Cache {
@@ -81,9 +82,11 @@ struct Cache {
 
     int pages_for(int len) const { return (len + page_size - 1) / page_size; }
     // the first page a sequence of this length still reads: its next token, at position len, sees keys from
-    // len - window + 1 on
+    // len - window + 1 on, and from the start of its own block of `chunk` positions on
     int first_needed(const Group& g, int len) const {
-        return g.window > 0 ? std::max(0, len - g.window + 1) / page_size : 0;
+        int first = g.window > 0 ? std::max(0, len - g.window + 1) : 0;
+        if (g.chunk > 0) first = std::max(first, len / g.chunk * g.chunk);
+        return first / page_size;
     }
 };
 
@@ -93,7 +96,7 @@ extern "C" {
 
 const char* ptah_last_error() { return g_error.c_str(); }
 
-int ptah_abi_version() { return 4; }
+int ptah_abi_version() { return 5; }
 
 void* ptah_cache_new(int max_slots, int page_size, int n_groups, const int* group_pages, const int* group_windows) {
     if (max_slots <= 0 || page_size <= 0 || n_groups < 0) {
@@ -111,6 +114,17 @@ void* ptah_cache_new(int max_slots, int page_size, int n_groups, const int* grou
         c->groups[g].window = group_windows ? std::max(0, group_windows[g]) : 0;
     }
     return c;
+}
+
+// A group whose tokens see the keys of their own block of `chunk` positions only (blocks counted from a sequence's
+// start) gives the pages that lie wholly before a sequence's current block back to its pool, as a window does with the
+// pages it has left behind.  To be called before any slot is handed out.
+int ptah_cache_set_chunk(void* h, int group, int chunk) {
+    Cache* c = static_cast<Cache*>(h);
+    if (group < 0 || group >= (int)c->groups.size() || chunk < 0)
+        return fail(ERR_CACHE, "cache: group %d of %zu, chunk %d", group, c->groups.size(), chunk);
+    c->groups[group].chunk = chunk;
+    return OK;
 }
 
 void ptah_cache_delete(void* h) { delete static_cast<Cache*>(h); }
@@ -170,7 +184,7 @@ int ptah_reserve(void* h, int n, const int* slots, const int* new_tokens) {
     // pages that a window has left behind go back to the pool first: no later step reads them, whether
     // this one is accepted or not
     for (Group& gr : c->groups) {
-        if (gr.window <= 0) continue;
+        if (gr.window <= 0 && gr.chunk <= 0) continue;
         for (int i = 0; i < n; ++i) {
             std::vector<int>& l = gr.lists[slots[i]];
             const int keep_from = std::min((int)l.size(), c->first_needed(gr, c->length[slots[i]]));

@@ -11,7 +11,8 @@ The head is the embedding table on the final norm's output.
 Tensor names: ``embed``, ``final.norm``, and per layer i ``l<i>.norm1``, ``l<i>.norm2``, ``l<i>.shift``,
 ``l<i>.mix.<name>``, ``l<i>.mlp.<name>``.
 
-Storage per sequence: attention passes with equal kv heads and page head size share a page pool; linear-attention
+Storage per sequence: attention passes with equal kv heads, page head size and mask share a page pool (of a masked
+layer, a sequence holds the pages of its current block only); linear-attention
 passes with equal state sizes share a state table; the token-shift rows of all passes are one state table.
 """
 from __future__ import annotations
@@ -23,7 +24,7 @@ from ..config.registry import register
 from ..parts import (DecayLinearAttentionMixer, Embedding, GatedAttentionMixer, GatedFeedForward, NoPositions, OutputHead,
                      RMSNorm, RotaryPositions, RoutedFeedForward, ShiftedParallelBlock)
 from ..parts.positions import yarn_ramp_frequencies
-from .spec import CACHE_FULL, CACHE_STATE, CacheGroupSpec, LayerCall, ModelSpec
+from .spec import CACHE_CHUNK, CACHE_FULL, CACHE_STATE, CacheGroupSpec, LayerCall, ModelSpec
 
 GATE_ALPHA = 1.702  # the dense feed-forward's gate is g * sigmoid(1.702 g)
 
@@ -72,7 +73,7 @@ def build_bimepel(cfg: BimepelConfig) -> ModelSpec:
     for run, i in enumerate(cfg.run_order()):
         mixer = blocks[i].mixer
         if isinstance(mixer, GatedAttentionMixer):
-            key = ("kv", (mixer.kv_heads, mixer.frame))
+            key = ("kv", (mixer.kv_heads, mixer.frame, mixer.chunk))
         else:
             key = ("state", mixer.state_shape)
         entry = groups.setdefault(key, [f"{key[0]}{len(groups)}", 0])
@@ -80,8 +81,9 @@ def build_bimepel(cfg: BimepelConfig) -> ModelSpec:
         entry[1] += 1
     cache_groups = [CacheGroupSpec("shift", CACHE_STATE, len(order), state_shape=(H,))]
     for (kind, shape), (name, count) in groups.items():
-        if kind == "kv":
-            cache_groups.append(CacheGroupSpec(name, CACHE_FULL, count, shape[0], shape[1]))
+        if kind == "kv":  # a masked layer's pages behind its sequence's current block go back to the pool
+            cache_groups.append(CacheGroupSpec(name, CACHE_CHUNK if shape[2] else CACHE_FULL, count, shape[0], shape[1],
+                                               chunk=shape[2] or None))
         else:
             cache_groups.append(CacheGroupSpec(name, CACHE_STATE, count, state_shape=shape))
     return ModelSpec(

@@ -42,6 +42,7 @@ class TensorSpec:
 # kinds of per-sequence storage a group of layers can ask for
 CACHE_FULL = "full"  # every key and value of the sequence
 CACHE_WINDOW = "window"  # the last `window` keys and values
+CACHE_CHUNK = "chunk"  # the keys and values of the block of `chunk` positions that the sequence's next token lies in
 CACHE_STATE = "state"  # a tensor of fixed shape per sequence, zero at the sequence's start
 
 
@@ -55,6 +56,7 @@ class CacheGroupSpec:
     kv_heads: int = 0
     head_dim: int = 0
     window: Optional[int] = None
+    chunk: Optional[int] = None
     #: False: the group keeps no value pool (its layers read their values out of the key rows)
     values: bool = True
     state_shape: Tuple[int, ...] = ()

@@ -12,7 +12,7 @@ import os
 import threading
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-ABI_VERSION = 4
+ABI_VERSION = 5
 OK, ERR_STEP, ERR_CACHE, ERR_FULL = 0, 1, 2, 3
 
 _lib = None
@@ -43,6 +43,7 @@ def load():
         lib.ptah_cache_new.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, _P_INT, _P_INT]
         lib.ptah_cache_delete.argtypes = [ctypes.c_void_p]
         lib.ptah_cache_delete.restype = None
+        lib.ptah_cache_set_chunk.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int]
         for name in ("ptah_alloc", "ptah_free_slots", "ptah_check"):
             getattr(lib, name).argtypes = [ctypes.c_void_p]
         for name in ("ptah_free", "ptah_is_live", "ptah_length", "ptah_free_pages", "ptah_held_pages"):

@@ -75,7 +75,8 @@ def test_tensor_names_and_storage_of_every_pass():
     assert len({(c.cache_group, c.cache_layer) for c in spec.order}) == 7
     groups = {g.name: g for g in spec.cache_groups}
     assert groups["shift"].num_layers == 7 and groups["shift"].state_shape == (32,)
-    kv = sorted((g.kv_heads, g.head_dim, g.num_layers) for g in groups.values() if g.kind == "full")
-    assert kv == [(1, 32, 2), (2, 32, 2)]
+    # the masked attention's pages are a group that gives back what lies before a sequence's current block
+    kv = sorted((g.kind, g.kv_heads, g.head_dim, g.chunk, g.num_layers) for g in groups.values() if g.kind in ("full", "chunk"))
+    assert kv == [("chunk", 2, 32, 40, 2), ("full", 1, 32, None, 2)]
     states = sorted((g.state_shape, g.num_layers) for g in groups.values() if g.kind == "state" and g.name != "shift")
     assert states == [((96,), 1), ((192,), 2)]

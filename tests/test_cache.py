@@ -5,7 +5,7 @@ import pytest
 import torch
 
 from pytorch_transformers_amd.cache import CacheError, CacheFull, PagedCache
-from pytorch_transformers_amd.engine.spec import CACHE_FULL, CACHE_STATE, CACHE_WINDOW, CacheGroupSpec
+from pytorch_transformers_amd.engine.spec import CACHE_CHUNK, CACHE_FULL, CACHE_STATE, CACHE_WINDOW, CacheGroupSpec
 from pytorch_transformers_amd.engine.step import StepError, plan_step
 
 KV = CacheGroupSpec("kv", CACHE_FULL, num_layers=2, kv_heads=2, head_dim=16)
@@ -183,3 +183,31 @@ def test_a_window_group_gives_back_the_pages_behind_its_window():
     c.free(s); c.free(t)
     assert c.free_pages("near") == 16 and c.free_pages("kv") == 16
     c.check_consistent()
+
+
+def test_a_chunk_group_gives_back_the_pages_before_its_current_block():
+    """A group whose tokens see their own block of 100 positions holds the pages from that block's start on, however
+    long the sequence grows, also when a prompt comes in portions that end inside a block."""
+    c = _cache(64 * 16, groups=(KV, CacheGroupSpec("block", CACHE_CHUNK, 1, 1, 16, chunk=100)), max_slots=2)
+    s = c.alloc()
+    c.reserve([s], [250]); c.commit([s], [250])  # a prompt needs all its pages while it runs: its tokens lie in three blocks
+    assert c.page_list("block", s) == [0, 1, 2, 3]
+    c.reserve([s], [30])  # the next token, at 250, lies in the block that starts at 200: pages 0..2 (positions 0..191) are before it
+    # (the new page is one that just came back: lowest first)
+    assert c.page_list("block", s) == [-1, -1, -1, 3, 0] and c.page_list("kv", s) == [0, 1, 2, 3, 4]
+    c.commit([s], [30]); c.check_consistent()
+    for _ in range(20):  # 280 .. 299 stay in the block, 300 starts one: page 3 (192..255) goes, page 4 (256..319) stays
+        c.reserve([s], [1]); c.commit([s], [1])
+    assert c.page_list("block", s) == [-1, -1, -1, 3, 0]
+    c.reserve([s], [1]); c.commit([s], [1])
+    assert c.page_list("block", s) == [-1, -1, -1, -1, 0] and c.length(s) == 301
+    for _ in range(400):
+        c.reserve([s], [1]); c.commit([s], [1])
+    c.check_consistent()
+    held = [p for p in c.page_list("block", s) if p >= 0]
+    assert 1 <= len(held) <= 3 and c.page_list("block", s)[-1] >= 0 and len(c.page_list("kv", s)) == 11
+    c.free(s)
+    assert c.free_pages("block") == 16 and c.free_pages("kv") == 16
+    c.check_consistent()
+    with pytest.raises(CacheError, match="positive block size"):
+        _cache(groups=(CacheGroupSpec("block", CACHE_CHUNK, 1, 1, 16),))
