@@ -92,7 +92,8 @@ class RMSNorm(Part):
 
     def forward_wide(self, x, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         """The norm of a ``WideResidual``'s 32-bit side, in its compute type."""
-        return self.apply(x.wide, x.narrow.dtype, rows=rows)[0]
+        dtype = getattr(x, "dtype", None) or x.narrow.dtype  # (a sum that is not formed says its compute type itself)
+        return self.apply(x.wide, dtype, rows=rows)[0]
 
 
 register_part("norm", "layernorm", LayerNorm)
